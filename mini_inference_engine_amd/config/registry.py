@@ -75,9 +75,9 @@ def _ensure_builtin() -> None:
 
 
 def architecture_for(config: Mapping[str, Any]) -> Architecture:
-    """Choose by ``architectures[0]``; fall back on ``model_type``."""
+    """Choose by ``architectures[0]`` (or the single name under ``architecture``); fall back on ``model_type``."""
     _ensure_builtin()
-    names = config.get("architectures") or []
+    names = config.get("architectures") or config.get("architecture") or []
     if isinstance(names, str):
         names = [names]
     for n in names:

@@ -12,6 +12,9 @@ from dataclasses import dataclass
 from typing import Any
 
 
+ACTIVATIONS = ("silu", "gelu_tanh", "relu2")
+
+
 @dataclass
 class Sink:
     """Where a part's last product goes: added into the float32 ``stream``; and, if the block knows it,
@@ -49,6 +52,14 @@ class Normed:
         return self._value
 
 
+class StreamCopy:
+    """The residual stream as it stands, in the activation dtype (``value``; the stream itself where that is
+    float32): what a block hands on when nothing is pending and its branches read the stream unnormed."""
+
+    def __init__(self, stream, value):
+        self.stream, self.value = stream, value
+
+
 class KernelBackend:
     name = "?"
     act_dtype = None
@@ -57,8 +68,8 @@ class KernelBackend:
         """Row counts of steps that will recur (the batch sizes decode graphs are captured at, the token budget
         of a step): a backend may spend time once, outside any capture, to choose its kernels for them."""
 
-    def embedding(self, ids, table, taken_from=None, earlier_tokens=None):
-        """stream[t, :] = float(table[ids[t], :]) -> [T, width] float32.  With ``taken_from`` (int32 [T]):
+    def embedding(self, ids, table, taken_from=None, earlier_tokens=None, scale=1.0):
+        """stream[t, :] = float(table[ids[t], :]) * scale -> [T, width] float32.  With ``taken_from`` (int32 [T]):
         where it is >= 0 the token is ``earlier_tokens[taken_from[t]]`` instead of ``ids[t]`` (a token the
         step before chose, read on the device because the host has not seen it yet)."""
         raise NotImplementedError
@@ -80,6 +91,81 @@ class KernelBackend:
     def linear_silu_mul(self, x, w_gate_up, intermediate):
         """gu = x w^T with w [2 * intermediate, in]; returns silu(gu[:, :I]) * gu[:, I:].
         ``x`` is a tensor or a Normed."""
+        raise NotImplementedError
+
+    def linear_act_mul(self, x, w_gate_up, intermediate, activation="silu"):
+        """The same with another gate function: act(gu[:, :I]) * gu[:, I:], act one of ACTIVATIONS."""
+        if activation == "silu":
+            return self.linear_silu_mul(x, w_gate_up, intermediate)
+        raise NotImplementedError
+
+    def scale_(self, t, factor):
+        """t *= factor in place (float32), returns t."""
+        raise NotImplementedError
+
+    def branch_norm_add(self, y, stream, weight, eps):
+        """stream += y * rsqrt(mean(y^2) + eps) * weight, row by row in float32 (y [T, width] of any float
+        dtype; None: nothing is added).  Returns the updated stream in the activation dtype, rounded once
+        (the stream itself where that is float32)."""
+        raise NotImplementedError
+
+    def rmsnorm_columns(self, x, col, n, weight, eps):
+        """RMSNorm of columns [col, col + n) of x [T, *] float32, times weight [n] -> [T, n] in the activation dtype."""
+        raise NotImplementedError
+
+    # ---- attention through a cached latent (one shared latent "head" of kv_rank + rot_dim numbers a token)
+    def latent_kv_store(self, sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache,
+                        slot_mapping):
+        """Columns [col, col + kv_rank + rot_dim) of ``sums`` [T, *] float32 are a token's down-projection.  The
+        first kv_rank, RMS-normed with ``norm_weight``, are its latent c; of the last rot_dim the first
+        2 * len(inv_freq) turn in adjacent pairs (2i, 2i + 1) by the angle position * inv_freq[i] (32-bit).
+        Token t's slot of k_cache [pages, 1, page, P] gets [c | turned part | zeros], of v_cache [pages, 1, P, page]
+        [c | zeros] (P = the cache's padded size >= kv_rank + rot_dim)."""
+        raise NotImplementedError
+
+    def latent_query(self, q, w_uk, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim):
+        """q [T, H (dim + rot_dim)]; w_uk [H dim, kv_rank].  Per head h: [q_h[:dim] W_uk,h | turned q_h[dim:] | zeros]
+        -> [T, H padded_dim] in the activation dtype: the query against a cached latent, since
+        q_h[:dim] . (W_uk,h c) = (q_h[:dim] W_uk,h) . c."""
+        raise NotImplementedError
+
+    def latent_value_gate(self, o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim):
+        """o [T, H padded_dim] (attention over the latents; the first kv_rank of each head count); w_uv [H vdim,
+        kv_rank]; gate [T, *] float32 whose columns [gate_col, gate_col + H vdim) are the gate before its sigmoid.
+        -> (W_uv,h o_h) * sigmoid(gate) [T, H vdim] in the activation dtype."""
+        raise NotImplementedError
+
+    # ---- gated linear recurrence with a short convolution before it
+    def causal_conv(self, x, col, channels, in_bias, taps, conv_bias, tail, step):
+        """u[t, c] = conv_bias[c] + sum_k taps[c, k] * in(t - (K - 1 - k), c), in(t, c) = x[t, col + c] + in_bias[c]
+        (x float32 [T, *]); inputs before a row's first token come from ``tail`` [slots, K - 1, channels] float32
+        (the last K - 1 inputs of the row's request, zeros at its start), which this call only reads.
+        -> [T, channels] float32."""
+        raise NotImplementedError
+
+    def grouped_linear(self, x, w, bias=None, x_groups=None):
+        """x [T, Gx * in] float; w [G, out, in]; bias [G, out] or None.  Group g multiplies block g % Gx of x's
+        columns (x_groups = Gx, default G): y[t, g, :] = w[g] x[t, g % Gx, :] + bias[g] -> [T, G * out] float32,
+        32-bit arithmetic throughout."""
+        raise NotImplementedError
+
+    def rglru_scan(self, u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, step, decay_scale=8.0):
+        """Per row and channel, tokens in order: r, i = sigmoid of gates[t, c], gates[t, C + c];
+        a = exp(-decay_scale * r * softplus(lam[c])); S = a S + sqrt(1 - a^2) * i * u[t, c] from the row's slot of
+        ``state`` [slots, C] float32, left there afterwards; out[t, c] = S * gelu_tanh(y[t, y_col + c] + y_bias[c]).
+        Also shifts the row's inputs x[t, x_col + c] + x_bias[c] into ``tail`` [slots, K - 1, C].  All float32;
+        -> [T, C] in the activation dtype."""
+        raise NotImplementedError
+
+    # ---- routed experts
+    def route_topk(self, logits, bias, top):
+        """logits [T, E] float32 (+ bias [E]): the ``top`` largest of a token (lowest index first among equals), in
+        falling order, and the softmax over those alone -> (experts [T, top] int32, shares [T, top] float32)."""
+        raise NotImplementedError
+
+    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2"):
+        """y[t] = sum_j shares[t, j] * W_down[e] act(W_up[e] x[t]), e = experts[t, j]; w_up [E, ff, width],
+        w_down [E, width, ff]; the hidden activation is rounded once to the activation dtype -> [T, width] float32."""
         raise NotImplementedError
 
     def rotary_kv_store(self, qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,

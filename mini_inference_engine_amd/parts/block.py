@@ -7,7 +7,7 @@ be added: the next block's first norm (or the final norm) adds it
 """
 from __future__ import annotations
 
-from ..kernels.api import Sink
+from ..kernels.api import Normed, Sink, StreamCopy
 from .base import Block, register_block
 
 
@@ -44,3 +44,41 @@ def _sink(residual, norm):
     if weight is None or eps is None:
         return Sink(residual)
     return Sink(residual, weight, eps)
+
+
+@register_block("branch_norm")
+class BranchNormBlock(Block):
+    """The norm sits on each branch's output, and the branches read the stream itself:
+    stream += norm_mixer(mixer(stream)); stream += norm_feed_forward(feed_forward(stream)).  ``feed_forward``
+    (and its norm) may be None: the layer is its mixer alone.  Between the branches the stream travels in the
+    activation dtype beside its float32 self (kernels.api.StreamCopy), made by the kernel that adds a branch."""
+
+    def __init__(self, mixer, norm_mixer, feed_forward=None, norm_feed_forward=None):
+        if (feed_forward is None) != (norm_feed_forward is None):
+            raise ValueError("a feed-forward and its norm come together or not at all")
+        self.mixer = mixer
+        self.norm_mixer = norm_mixer
+        self.feed_forward = feed_forward
+        self.norm_feed_forward = norm_feed_forward
+
+    def children(self):
+        return [p for p in (self.mixer, self.norm_mixer, self.feed_forward, self.norm_feed_forward) if p is not None]
+
+    def forward(self, h, residual, step, cache, next_norm=None):
+        ops = self.ops
+        if isinstance(h, StreamCopy) and h.stream is residual:
+            x = h.value
+        else:
+            if isinstance(h, Normed):         # a block of another kind before this one: its last add may be pending
+                h, h_pending = None, h.pending
+                if h_pending is not None:
+                    residual.add_(h_pending.float())
+            elif h is not None:
+                residual.add_(h.float())
+            x = ops.branch_norm_add(None, residual, None, 0.0)
+        y = self.mixer.forward(x, step, cache)
+        x = ops.branch_norm_add(y, residual, self.norm_mixer.weight, self.norm_mixer.eps)
+        if self.feed_forward is not None:
+            y = self.feed_forward.forward(x, step)
+            x = ops.branch_norm_add(y, residual, self.norm_feed_forward.weight, self.norm_feed_forward.eps)
+        return StreamCopy(residual, x), residual

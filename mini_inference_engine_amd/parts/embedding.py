@@ -1,8 +1,8 @@
 """Token embedding and output head.
 
-stream[t] = E[id[t]], unscaled, no position term (inference_engine/model.py:96,168);
-logits = y W_lm^T with W_lm = E when tied (inference_engine/model.py:112-113,185).
-The stream is 32-bit; logits come out in 32-bit.
+stream[t] = E[id[t]] * scale (scale 1 by default), no position term (inference_engine/model.py:96,168);
+logits = y W_lm^T * scale with W_lm = E when tied (inference_engine/model.py:112-113,185; the tied
+table is used as stored, without the embedding's scale).  The stream is 32-bit; logits come out in 32-bit.
 """
 from __future__ import annotations
 
@@ -12,10 +12,11 @@ from .base import ParamSpec, Part
 
 
 class Embedding(Part):
-    def __init__(self, vocab_size: int, width: int, weight_name: str):
+    def __init__(self, vocab_size: int, width: int, weight_name: str, scale: float = 1.0):
         self.vocab_size = int(vocab_size)
         self.width = int(width)
         self.weight_name = weight_name
+        self.scale = float(scale)
         self.weight = None
 
     def params(self):
@@ -23,11 +24,15 @@ class Embedding(Part):
 
     def forward(self, ids, taken_from=None, earlier_tokens=None):
         """``taken_from`` / ``earlier_tokens``: see KernelBackend.embedding (tokens still on the device)."""
+        if self.scale != 1.0:
+            return self.ops.embedding(ids, self.weight, taken_from, earlier_tokens, scale=self.scale)
         return self.ops.embedding(ids, self.weight, taken_from, earlier_tokens)
 
 
 class LMHead(Part):
-    def __init__(self, vocab_size: int, width: int, weight_name: str, tied_to: Embedding | None = None):
+    def __init__(self, vocab_size: int, width: int, weight_name: str, tied_to: Embedding | None = None,
+                 scale: float = 1.0):
+        self.scale = float(scale)
         self.vocab_size = int(vocab_size)
         self.width = int(width)
         self.weight_name = weight_name
@@ -44,4 +49,5 @@ class LMHead(Part):
         return self.tied_to.weight if self.tied_to is not None else self._weight
 
     def forward(self, y):
-        return self.ops.linear(y, self.weight, out_dtype=torch.float32)
+        logits = self.ops.linear(y, self.weight, out_dtype=torch.float32)
+        return logits if self.scale == 1.0 else self.ops.scale_(logits, self.scale)

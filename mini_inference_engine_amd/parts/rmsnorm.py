@@ -7,7 +7,7 @@ The stream and every intermediate are 32-bit; y is rounded once.
 """
 from __future__ import annotations
 
-from ..kernels.api import Normed
+from ..kernels.api import Normed, StreamCopy
 from .base import Norm, ParamSpec, register_norm
 
 
@@ -29,9 +29,11 @@ class RMSNorm(Norm):
             if x.weight is self.weight and x.residual is residual and x.eps == self.eps and x.pending is None:
                 return x if rows is None else x.with_rows(rows)
             x = None
+        if isinstance(x, StreamCopy):       # the block before left nothing pending
+            x = None
         return Normed(self.ops, x, residual, self.weight, self.eps, rows)
 
     def forward(self, x, residual, rows=None, out_dtype=None):
-        if isinstance(x, Normed):
+        if isinstance(x, (Normed, StreamCopy)):
             return self.lazy(x, residual, rows).materialize(out_dtype)
         return self.ops.add_rmsnorm(x, residual, self.weight, self.eps, out_dtype=out_dtype, rows=rows)

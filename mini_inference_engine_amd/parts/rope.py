@@ -68,3 +68,25 @@ class NoPosition(PositionEncoding):
     def project_encode_store(self, ops, x, w_qkv, step, num_q_heads, num_kv_heads, k_cache, v_cache, slots):
         return ops.linear_rotary_kv_store(x, w_qkv, step.positions, None, None, 0, num_q_heads, num_kv_heads,
                                           self.head_dim, k_cache, v_cache, slots, for_attention=True)
+
+
+@register_position_encoding("rotary_interleaved")
+class RotaryInterleaved(PositionEncoding):
+    """Adjacent pairs: elements 2i and 2i + 1 of the first ``rotary_dim`` dims turn together by the angle
+    position * theta^(-2i / rotary_dim); (u, v) -> (u cos - v sin, v cos + u sin).  The kernels that use it
+    compute the angle and its cosine and sine in 32-bit from the position and ``inv_freq`` [rotary_dim / 2]
+    themselves, so there is no table and no longest position."""
+
+    def __init__(self, rotary_dim: int, theta: float):
+        self.rotary_dim = int(rotary_dim)
+        self.theta = float(theta)
+        if self.rotary_dim % 2 or self.rotary_dim < 2:
+            raise ValueError(f"rotary_dim {self.rotary_dim} must be even and at least 2")
+        if not self.theta > 0:
+            raise ValueError("theta must be positive")
+        self.inv_freq = None
+
+    def prepare(self, device, dtype):
+        if self.inv_freq is None or self.inv_freq.device != torch.device(device):
+            exponent = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64) / self.rotary_dim
+            self.inv_freq = (self.theta ** -exponent).to(torch.float32).to(device).contiguous()

@@ -15,8 +15,132 @@ import torch
 from mini_inference_engine_amd.kernels.api import KernelBackend, Normed, Sink
 
 
-def ref_embedding(ids, table):
-    return table[ids.long()].float()
+def ref_embedding(ids, table, scale=1.0):
+    out = table[ids.long()].float()
+    return out if scale == 1.0 else out * scale
+
+
+def ref_act(z, activation):
+    if activation == "silu":
+        return z * torch.sigmoid(z)
+    if activation == "gelu_tanh":
+        return 0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+    if activation == "relu2":
+        return torch.relu(z) ** 2
+    raise ValueError(activation)
+
+
+def ref_branch_norm_add(y, stream, weight, eps, act_dtype):
+    if y is not None:
+        yd = y.double()
+        stream.add_((yd * torch.rsqrt(yd.pow(2).mean(-1, keepdim=True) + eps) * weight.double()).float())
+    return stream if act_dtype == torch.float32 else stream.to(act_dtype)
+
+
+def ref_rmsnorm_columns(x, col, n, weight, eps, out_dtype):
+    xd = x[:, col:col + n].double()
+    return (xd * torch.rsqrt(xd.pow(2).mean(-1, keepdim=True) + eps) * weight.double()).to(out_dtype)
+
+
+def ref_turn_pairs(x, positions, inv_freq):
+    """x [T, heads, d] float64: the first 2 * len(inv_freq) dims turn in adjacent pairs; the angle is a float32 product."""
+    n = 2 * inv_freq.shape[0]
+    angle = (positions.float()[:, None] * inv_freq.float()[None, :]).double()
+    c, s = angle.cos()[:, None, :], angle.sin()[:, None, :]
+    u, v = x[..., 0:n:2], x[..., 1:n:2]
+    out = x.clone()
+    out[..., 0:n:2] = u * c - v * s
+    out[..., 1:n:2] = v * c + u * s
+    return out
+
+
+def ref_latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache, slots):
+    P = k_cache.shape[2]
+    c = ref_rmsnorm_columns(sums, col, kv_rank, norm_weight, eps, torch.float64)
+    kr = ref_turn_pairs(sums[:, None, col + kv_rank:col + kv_rank + rot_dim].double(), positions, inv_freq)[:, 0]
+    page, off = slots.long() // P, slots.long() % P
+    k_cache[page, 0, off, :] = 0
+    k_cache[page, 0, off, :kv_rank] = c.to(k_cache.dtype)
+    k_cache[page, 0, off, kv_rank:kv_rank + rot_dim] = kr.to(k_cache.dtype)
+    v_cache[page, 0, :, off] = 0
+    v_cache[page, 0, :kv_rank, off] = c.to(v_cache.dtype)
+
+
+def ref_latent_query(q, w_uk, H, dim, rot_dim, kv_rank, positions, inv_freq, padded, out_dtype):
+    T = q.shape[0]
+    qh = q.double().view(T, H, dim + rot_dim)
+    out = torch.zeros(T, H, padded, dtype=torch.float64, device=q.device)
+    out[..., :kv_rank] = torch.einsum("thd,hdr->thr", qh[..., :dim], w_uk.double().view(H, dim, kv_rank))
+    out[..., kv_rank:kv_rank + rot_dim] = ref_turn_pairs(qh[..., dim:], positions, inv_freq)
+    return out.view(T, H * padded).to(out_dtype)
+
+
+def ref_latent_value_gate(o, w_uv, gate, gate_col, H, vdim, kv_rank, padded, out_dtype):
+    T = o.shape[0]
+    v = torch.einsum("thr,hvr->thv", o.double().view(T, H, padded)[..., :kv_rank], w_uv.double().view(H, vdim, kv_rank))
+    v = v.reshape(T, H * vdim)
+    if gate is not None:
+        v = v * torch.sigmoid(gate[:, gate_col:gate_col + H * vdim].double())
+    return v.to(out_dtype)
+
+
+def ref_causal_conv(x, col, C, in_bias, taps, conv_bias, tail, row_start, slots):
+    K = taps.shape[1]
+    out = torch.empty(x.shape[0], C, dtype=torch.float32, device=x.device)
+    for r in range(len(slots)):
+        a, b = int(row_start[r]), int(row_start[r + 1])
+        inp = torch.cat([tail[int(slots[r])][:K - 1].double(), x[a:b, col:col + C].double() + in_bias.double()])
+        acc = conv_bias.double().expand(b - a, C).clone()
+        for k in range(K):
+            acc += inp[k:k + b - a] * taps[:, k].double()
+        out[a:b] = acc.float()
+    return out
+
+
+def ref_grouped_linear(x, w, bias, x_groups):
+    G, n_out, n_in = w.shape
+    gx = x_groups or G
+    xb = x.double().view(x.shape[0], gx, n_in)
+    y = torch.stack([xb[:, g % gx] @ w[g].double().T for g in range(G)], 1)
+    if bias is not None:
+        y = y + bias.double().view(1, G, n_out)
+    return y.reshape(x.shape[0], G * n_out).float()
+
+
+def ref_rglru_scan(u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, row_start, slots, decay_scale, out_dtype):
+    C = u.shape[1]
+    K1 = tail.shape[1]
+    out = torch.empty(u.shape[0], C, dtype=torch.float64, device=u.device)
+    sp = torch.nn.functional.softplus(lam.double())
+    for r in range(len(slots)):
+        a0, b0, slot = int(row_start[r]), int(row_start[r + 1]), int(slots[r])
+        S = state[slot].double()
+        for t in range(a0, b0):
+            rg, ig = torch.sigmoid(gates[t, :C].double()), torch.sigmoid(gates[t, C:].double())
+            a = torch.exp(-decay_scale * rg * sp)
+            S = a * S + torch.sqrt(1.0 - a * a) * ig * u[t].double()
+            out[t] = S * ref_act(y[t, y_col:y_col + C].double() + y_bias.double(), "gelu_tanh")
+        state[slot] = S.float()
+        inp = torch.cat([tail[slot].double(), x[a0:b0, x_col:x_col + C].double() + x_bias.double()])
+        tail[slot] = inp[-K1:].float()
+    return out.to(out_dtype)
+
+
+def ref_route_topk(logits, bias, top):
+    z = logits.double() if bias is None else logits.double() + bias.double()
+    order = torch.sort(z, dim=-1, descending=True, stable=True)
+    idx, val = order.indices[:, :top], order.values[:, :top]
+    return idx.to(torch.int32), torch.softmax(val, -1).float()
+
+
+def ref_routed_experts(x, experts, shares, w_up, w_down, activation, act_dtype):
+    y = torch.zeros(x.shape[0], w_down.shape[1], dtype=torch.float64, device=x.device)
+    for t in range(x.shape[0]):
+        for j in range(experts.shape[1]):
+            e = int(experts[t, j])
+            h = ref_act(x[t].double() @ w_up[e].double().T, activation).to(act_dtype).double()
+            y[t] += shares[t, j].double() * (h @ w_down[e].double().T)
+    return y.float()
 
 
 def ref_add_rmsnorm(x, residual, weight, eps, out_dtype, rows=None):
@@ -131,11 +255,58 @@ class TorchBackend(KernelBackend):
     def _count(self, name):
         self.calls[name] = self.calls.get(name, 0) + 1
 
-    def embedding(self, ids, table, taken_from=None, earlier_tokens=None):
+    def embedding(self, ids, table, taken_from=None, earlier_tokens=None, scale=1.0):
         self._count("embedding")
         if taken_from is not None:
             ids = torch.where(taken_from >= 0, earlier_tokens[taken_from.clamp(min=0).long()], ids)
-        return ref_embedding(ids, table)
+        return ref_embedding(ids, table, scale)
+
+    def scale_(self, t, factor):
+        return t.mul_(factor)
+
+    def branch_norm_add(self, y, stream, weight, eps):
+        self._count("branch_norm_add")
+        return ref_branch_norm_add(y, stream, weight, eps, self.act_dtype)
+
+    def rmsnorm_columns(self, x, col, n, weight, eps):
+        return ref_rmsnorm_columns(x, col, n, weight, eps, self.act_dtype)
+
+    def linear_act_mul(self, x, w_gate_up, intermediate, activation="silu"):
+        self._count("linear_act_mul")
+        if isinstance(x, Normed):
+            x = x.materialize()
+        gu = ref_linear(x, w_gate_up, None, self.act_dtype).double()
+        return (ref_act(gu[:, :intermediate], activation) * gu[:, intermediate:]).to(self.act_dtype)
+
+    def latent_kv_store(self, sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache,
+                        slot_mapping):
+        self._count("latent_kv_store")
+        ref_latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache, slot_mapping)
+
+    def latent_query(self, q, w_uk, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim):
+        return ref_latent_query(q, w_uk, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim, self.act_dtype)
+
+    def latent_value_gate(self, o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim):
+        return ref_latent_value_gate(o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim, self.act_dtype)
+
+    def causal_conv(self, x, col, channels, in_bias, taps, conv_bias, tail, step):
+        return ref_causal_conv(x, col, channels, in_bias, taps, conv_bias, tail, step.host["row_start"],
+                               step.host["state_slots"])
+
+    def grouped_linear(self, x, w, bias=None, x_groups=None):
+        return ref_grouped_linear(x, w, bias, x_groups)
+
+    def rglru_scan(self, u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, step, decay_scale=8.0):
+        self._count("rglru_scan")
+        return ref_rglru_scan(u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, step.host["row_start"],
+                              step.host["state_slots"], decay_scale, self.act_dtype)
+
+    def route_topk(self, logits, bias, top):
+        return ref_route_topk(logits, bias, top)
+
+    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2"):
+        self._count("routed_experts")
+        return ref_routed_experts(x, experts, shares, w_up, w_down, activation, self.act_dtype)
 
     def add_rmsnorm(self, x, residual, weight, eps, out_dtype=None, rows=None):
         self._count("add_rmsnorm")
