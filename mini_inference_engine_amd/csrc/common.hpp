@@ -75,6 +75,22 @@ __device__ __forceinline__ void rotate_pair(float x1, float x2, float c, float s
   o2 = fmaf(x2, c, x1 * s);
 }
 
+// ---- activation functions shared by the feed-forward kernels (codes shared with the Python side)
+enum { MIE_ACT_NONE = 0, MIE_ACT_SILU = 1, MIE_ACT_GELU_TANH = 2, MIE_ACT_RELU2 = 3 };
+
+__device__ __forceinline__ float mie_gelu_tanh(float z) {
+  return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+__device__ __forceinline__ float mie_act(float z, int act) {
+  switch (act) {
+    case MIE_ACT_SILU: return z / (1.0f + expf(-z));
+    case MIE_ACT_GELU_TANH: return mie_gelu_tanh(z);
+    case MIE_ACT_RELU2: { const float r = fmaxf(z, 0.f); return r * r; }
+    default: return z;
+  }
+}
+__device__ __forceinline__ float mie_sigmoid(float z) { return 1.0f / (1.0f + expf(-z)); }
+
 // ---- host-side error plumbing
 static thread_local char g_mie_error[512];
 #define MIE_FAIL(...)                                        \

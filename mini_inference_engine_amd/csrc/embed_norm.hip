@@ -1,6 +1,6 @@
 // Token embedding into the 32-bit residual stream, and the residual add fused with RMSNorm.
 //
-// embedding:    stream[t, :] = float(table[ids[t], :])
+// embedding:    stream[t, :] = float(table[ids[t], :]) * scale
 // add_rmsnorm:  r = stream[row] (+ float(x[row]));  stream[row] = r (unless rows are gathered);
 //               y[row] = r * (1 / sqrt(mean(r^2) + eps)) * weight, rounded once to y's type.
 // One workgroup per row; the row's sum of squares is reduced in an order that depends only on
@@ -10,7 +10,7 @@
 template <typename TT>
 __global__ void embedding_kernel(const int* __restrict__ ids, const TT* __restrict__ table, float* __restrict__ out,
                                  int width, int vocab, const int* __restrict__ taken_from,
-                                 const int* __restrict__ earlier_tokens) {
+                                 const int* __restrict__ earlier_tokens, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   if (taken_from) {            // a token the host does not know yet: entry taken_from[t] of the tokens chosen last
@@ -20,7 +20,7 @@ __global__ void embedding_kernel(const int* __restrict__ ids, const TT* __restri
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // ids are validated on the host; never read outside
   const TT* src = table + (size_t)id * width;
   float* dst = out + (size_t)t * width;
-  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float(src[i]);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = to_float(src[i]) * scale;
 }
 
 #define NORM_THREADS 256
@@ -166,17 +166,18 @@ MIE_EXPORT const char* embed_norm_last_error() { return g_mie_error; }
 // taken_from (or null) [tokens]: where >= 0, the token is earlier_tokens[taken_from[t]] instead of ids[t]
 // (a token chosen by the step before, which the host has not seen yet).
 MIE_EXPORT int mie_embedding(const int* ids, const void* table, int table_dtype, float* out, int tokens, int width,
-                             int vocab, const int* taken_from, const int* earlier_tokens, hipStream_t stream) {
+                             int vocab, const int* taken_from, const int* earlier_tokens, float scale,
+                             hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (width <= 0 || vocab <= 0) MIE_FAIL("embedding: width %d, vocab %d", width, vocab);
   if (taken_from && !earlier_tokens) MIE_FAIL("embedding: taken_from without the tokens to take from");
   dim3 grid(tokens), block(256);
   if (table_dtype == MIE_F32)
     hipLaunchKernelGGL(embedding_kernel<float>, grid, block, 0, stream, ids, (const float*)table, out, width, vocab,
-                       taken_from, earlier_tokens);
+                       taken_from, earlier_tokens, scale);
   else if (table_dtype == MIE_BF16)
     hipLaunchKernelGGL(embedding_kernel<bf16>, grid, block, 0, stream, ids, (const bf16*)table, out, width, vocab,
-                       taken_from, earlier_tokens);
+                       taken_from, earlier_tokens, scale);
   else
     MIE_FAIL("embedding: table dtype code %d", table_dtype);
   MIE_CHECK_LAUNCH("embedding");
@@ -227,4 +228,125 @@ MIE_EXPORT int mie_add_rmsnorm(const void* x, int x_dtype, float* stream, const 
   if (x_dtype == MIE_BF16 && w_dtype == MIE_F32) return launch_norm<bf16, float>(x, stream, weight, y, y_dtype, rows, n_rows, width, eps, s);
   if (x_dtype == MIE_BF16 && w_dtype == MIE_BF16) return launch_norm<bf16, bf16>(x, stream, weight, y, y_dtype, rows, n_rows, width, eps, s);
   MIE_FAIL("add_rmsnorm: dtype codes x %d, weight %d", x_dtype, w_dtype);
+}
+
+
+// ---- the norm on a branch's output: stream[row] += y[row] * (1 / sqrt(mean(y[row]^2) + eps)) * weight, in 32-bit,
+// and the updated stream once more in the activation dtype (copy; null where that is the stream itself).
+// y null: nothing is added, only the copy is made.  One workgroup a row, the same reduction order for every row.
+template <typename TY, typename TW, typename TO>
+__global__ void __launch_bounds__(NORM_THREADS)
+branch_norm_add_kernel(const TY* __restrict__ y, float* __restrict__ stream, const TW* __restrict__ weight,
+                       TO* __restrict__ copy, int width, float eps) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  float* sr = stream + (size_t)row * width;
+  TO* cr = copy ? copy + (size_t)row * width : nullptr;
+  if (!y) {
+    if (cr)
+      for (int i = threadIdx.x; i < width; i += NORM_THREADS) cr[i] = from_float<TO>(sr[i]);
+    return;
+  }
+  const TY* yr = y + (size_t)row * width;
+  float cache[NORM_CACHE];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < NORM_CACHE; ++k) {
+    const int i = threadIdx.x + k * NORM_THREADS;
+    const float v = i < width ? to_float(yr[i]) : 0.f;
+    cache[k] = v;
+    ss = fmaf(v, v, ss);
+  }
+  for (int i = threadIdx.x + NORM_CACHE * NORM_THREADS; i < width; i += NORM_THREADS) {
+    const float v = to_float(yr[i]);
+    ss = fmaf(v, v, ss);
+  }
+  const float rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+#pragma unroll
+  for (int k = 0; k < NORM_CACHE; ++k) {
+    const int i = threadIdx.x + k * NORM_THREADS;
+    if (i < width) {
+      const float r = sr[i] + cache[k] * rstd * to_float(weight[i]);
+      sr[i] = r;
+      if (cr) cr[i] = from_float<TO>(r);
+    }
+  }
+  for (int i = threadIdx.x + NORM_CACHE * NORM_THREADS; i < width; i += NORM_THREADS) {
+    const float r = sr[i] + to_float(yr[i]) * rstd * to_float(weight[i]);
+    sr[i] = r;
+    if (cr) cr[i] = from_float<TO>(r);
+  }
+}
+
+template <typename TY, typename TW>
+static int launch_branch_norm(const void* y, float* stream, const void* w, void* copy, int copy_dtype, int rows, int width,
+                              float eps, hipStream_t s) {
+  if (copy_dtype == MIE_BF16)
+    hipLaunchKernelGGL((branch_norm_add_kernel<TY, TW, bf16>), dim3(rows), dim3(NORM_THREADS), 0, s, (const TY*)y, stream,
+                       (const TW*)w, (bf16*)copy, width, eps);
+  else
+    hipLaunchKernelGGL((branch_norm_add_kernel<TY, TW, float>), dim3(rows), dim3(NORM_THREADS), 0, s, (const TY*)y, stream,
+                       (const TW*)w, (float*)copy, width, eps);
+  MIE_CHECK_LAUNCH("branch_norm_add");
+  return 0;
+}
+
+// y [rows, width] (or null), weight [width]; copy [rows, width] of copy_dtype, or null.
+MIE_EXPORT int mie_branch_norm_add(const void* y, int y_dtype, float* stream, const void* weight, int w_dtype, void* copy,
+                                   int copy_dtype, int rows, int width, float eps, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (width <= 0 || !stream) MIE_FAIL("branch_norm_add: width %d", width);
+  if (y && !weight) MIE_FAIL("branch_norm_add: a branch output without a norm weight");
+  if (!y && !copy) return 0;
+  if (copy && copy_dtype != MIE_F32 && copy_dtype != MIE_BF16) MIE_FAIL("branch_norm_add: copy dtype code %d", copy_dtype);
+  if (y_dtype == MIE_F32 && w_dtype == MIE_F32) return launch_branch_norm<float, float>(y, stream, weight, copy, copy_dtype, rows, width, eps, s);
+  if (y_dtype == MIE_F32 && w_dtype == MIE_BF16) return launch_branch_norm<float, bf16>(y, stream, weight, copy, copy_dtype, rows, width, eps, s);
+  if (y_dtype == MIE_BF16 && w_dtype == MIE_F32) return launch_branch_norm<bf16, float>(y, stream, weight, copy, copy_dtype, rows, width, eps, s);
+  if (y_dtype == MIE_BF16 && w_dtype == MIE_BF16) return launch_branch_norm<bf16, bf16>(y, stream, weight, copy, copy_dtype, rows, width, eps, s);
+  MIE_FAIL("branch_norm_add: dtype codes y %d, weight %d", y_dtype, w_dtype);
+}
+
+// ---- RMSNorm of a range of columns of a float32 matrix: out[row, i] = x[row, i] * rstd * weight[i], i < n
+template <typename TW, typename TO>
+__global__ void __launch_bounds__(NORM_THREADS)
+rmsnorm_columns_kernel(const float* __restrict__ x, long ldx, const TW* __restrict__ weight, TO* __restrict__ out, int n,
+                       float eps) {
+  __shared__ float scratch[16];
+  const float* xr = x + (size_t)blockIdx.x * ldx;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += NORM_THREADS) ss = fmaf(xr[i], xr[i], ss);
+  const float rstd = 1.0f / sqrtf(block_sum(ss, scratch) / (float)n + eps);
+  TO* o = out + (size_t)blockIdx.x * n;
+  for (int i = threadIdx.x; i < n; i += NORM_THREADS) o[i] = from_float<TO>(xr[i] * rstd * to_float(weight[i]));
+}
+
+// x points at the first column of the range; rows are ldx floats apart.
+MIE_EXPORT int mie_rmsnorm_columns(const float* x, long ldx, const void* weight, int w_dtype, void* out, int out_dtype,
+                                   int rows, int n, float eps, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (n <= 0 || ldx < n || !x || !weight || !out) MIE_FAIL("rmsnorm_columns: n %d, row stride %ld", n, ldx);
+#define RC_LAUNCH(TW_, TO_)                                                                                              \
+  hipLaunchKernelGGL((rmsnorm_columns_kernel<TW_, TO_>), dim3(rows), dim3(NORM_THREADS), 0, s, x, ldx, (const TW_*)weight, \
+                     (TO_*)out, n, eps)
+  if (w_dtype == MIE_F32 && out_dtype == MIE_F32) RC_LAUNCH(float, float);
+  else if (w_dtype == MIE_F32 && out_dtype == MIE_BF16) RC_LAUNCH(float, bf16);
+  else if (w_dtype == MIE_BF16 && out_dtype == MIE_F32) RC_LAUNCH(bf16, float);
+  else if (w_dtype == MIE_BF16 && out_dtype == MIE_BF16) RC_LAUNCH(bf16, bf16);
+  else MIE_FAIL("rmsnorm_columns: dtype codes weight %d, out %d", w_dtype, out_dtype);
+#undef RC_LAUNCH
+  MIE_CHECK_LAUNCH("rmsnorm_columns");
+  return 0;
+}
+
+// ---- t *= factor
+__global__ void scale_kernel(float* __restrict__ t, size_t n, float factor) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) t[i] *= factor;
+}
+
+MIE_EXPORT int mie_scale(float* t, long n, float factor, hipStream_t s) {
+  if (n <= 0) return 0;
+  long blocks = (n + 255) / 256;
+  hipLaunchKernelGGL(scale_kernel, dim3((unsigned)(blocks > 4096 ? 4096 : blocks)), dim3(256), 0, s, t, (size_t)n, factor);
+  MIE_CHECK_LAUNCH("scale");
+  return 0;
 }

@@ -82,6 +82,16 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, long ld_in, T* __restr
   }
 }
 
+// act(gate) * up for any of the activation codes of common.hpp
+template <typename T>
+__global__ void act_mul_kernel(const T* __restrict__ gu, long ld_in, T* __restrict__ out, long ld_out, int rows, int inter, int act) {
+  const size_t total = (size_t)rows * inter;
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t r = idx / inter, i = idx - r * inter;
+    out[r * ld_out + i] = from_float<T>(mie_act(to_float(gu[r * ld_in + i]), act) * to_float(gu[r * ld_in + inter + i]));
+  }
+}
+
 // bfloat16 rows whose gate and up halves start on 16 bytes: eight values a thread and a load
 __global__ void __launch_bounds__(256)
 silu_mul_bf16x8_kernel(const bf16* __restrict__ gu, long ld_in, bf16* __restrict__ out, long ld_out, int rows, int inter) {
@@ -158,5 +168,25 @@ MIE_EXPORT int mie_silu_mul(const void* gu, long ld_in, void* out, long ld_out, 
   else
     MIE_FAIL("silu_mul: dtype code %d", dtype);
   MIE_CHECK_LAUNCH("silu_mul");
+  return 0;
+}
+
+// The same with the gate's function chosen by code (common.hpp); silu takes the kernels above.
+MIE_EXPORT int mie_act_mul(const void* gu, long ld_in, void* out, long ld_out, int dtype, int rows, int inter, int act,
+                           hipStream_t s) {
+  if (act == MIE_ACT_SILU) return mie_silu_mul(gu, ld_in, out, ld_out, dtype, rows, inter, s);
+  if (rows <= 0 || inter <= 0) return 0;
+  if (act < MIE_ACT_NONE || act > MIE_ACT_RELU2) MIE_FAIL("act_mul: activation code %d", act);
+  if (ld_in < 2L * inter || ld_out < inter) MIE_FAIL("act_mul: leading dims %ld, %ld for intermediate %d", ld_in, ld_out, inter);
+  const size_t total = (size_t)rows * inter;
+  int blocks = (int)((total + 255) / 256);
+  if (blocks > 16384) blocks = 16384;
+  if (dtype == MIE_F32)
+    hipLaunchKernelGGL(act_mul_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, ld_in, (float*)out, ld_out, rows, inter, act);
+  else if (dtype == MIE_BF16)
+    hipLaunchKernelGGL(act_mul_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (const bf16*)gu, ld_in, (bf16*)out, ld_out, rows, inter, act);
+  else
+    MIE_FAIL("act_mul: dtype code %d", dtype);
+  MIE_CHECK_LAUNCH("act_mul");
   return 0;
 }

@@ -1,0 +1,102 @@
+// The gated linear recurrence of the recurrent mixer and the short causal convolution before it, over a step's
+// rows (a request's next tokens), with the request's state in its slot.  Everything is 32-bit.
+//
+// causal_conv:  u[t, c] = conv_bias[c] + sum_k taps[c, k] in(t - (K - 1 - k), c),  in(t, c) = x[t, c] + in_bias[c];
+//               inputs before the row's first token come from tail[slot] (the request's last K - 1 inputs, zeros at
+//               its start).  One thread a (token, channel); the tail is only read.
+// rglru_scan:   per (row, channel) thread, tokens in order:
+//                 r = sigmoid(gates[t, c]), i = sigmoid(gates[t, C + c]), a = exp(-decay_scale r softplus(lam[c])),
+//                 S = a S + sqrt(1 - a^2) i u[t, c];  out[t, c] = S gelu_tanh(y[t, c] + y_bias[c]);
+//               S starts from state[slot] and is left there; then the row's inputs are shifted into tail[slot].
+#include "common.hpp"
+
+__global__ void __launch_bounds__(256)
+causal_conv_kernel(const float* __restrict__ x, long ldx, const float* __restrict__ in_bias, const float* __restrict__ taps,
+                   const float* __restrict__ conv_bias, const float* __restrict__ tail, const int* __restrict__ token_row,
+                   const int* __restrict__ row_start, const int* __restrict__ slots, float* __restrict__ u, int C, int K) {
+  const int t = blockIdx.x;
+  const int r = token_row[t], j = t - row_start[r];
+  const float* tl = tail + (size_t)slots[r] * (K > 1 ? K - 1 : 1) * C;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
+    float acc = conv_bias[c];
+    const float b = in_bias[c];
+    for (int k = 0; k < K; ++k) {
+      const int back = K - 1 - k;              // how many tokens before t
+      const float v = back <= j ? x[(size_t)(t - back) * ldx + c] + b : tl[(size_t)(K - 1 + j - back) * C + c];
+      acc = fmaf(taps[(size_t)c * K + k], v, acc);
+    }
+    u[(size_t)t * C + c] = acc;
+  }
+}
+
+template <typename TO>
+__global__ void __launch_bounds__(256)
+rglru_scan_kernel(const float* __restrict__ u, const float* __restrict__ gates, const float* __restrict__ lam,
+                  const float* __restrict__ y, long ldy, const float* __restrict__ y_bias, const float* __restrict__ x,
+                  long ldx, const float* __restrict__ x_bias, float* __restrict__ state, float* __restrict__ tail,
+                  const int* __restrict__ row_start, const int* __restrict__ slots, TO* __restrict__ out, int C, int K,
+                  float decay_scale) {
+  const int r = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int a0 = row_start[r], b0 = row_start[r + 1], slot = slots[r];
+  const float lm = lam[c];
+  const float sp = decay_scale * (lm > 20.f ? lm : log1pf(expf(lm)));
+  const float yb = y_bias[c];
+  float S = state[(size_t)slot * C + c];
+  for (int t = a0; t < b0; ++t) {
+    const float rg = mie_sigmoid(gates[(size_t)t * 2 * C + c]);
+    const float ig = mie_sigmoid(gates[(size_t)t * 2 * C + C + c]);
+    const float log_a = -sp * rg;
+    const float a = expf(log_a);
+    // 1 - a^2 as -expm1(2 log a): no cancellation where a is close to 1
+    S = fmaf(a, S, sqrtf(-expm1f(2.0f * log_a)) * ig * u[(size_t)t * C + c]);
+    out[(size_t)t * C + c] = from_float<TO>(S * mie_gelu_tanh(y[(size_t)t * ldy + c] + yb));
+  }
+  state[(size_t)slot * C + c] = S;
+  // the last K - 1 of (old tail, this row's inputs), oldest first; reads run ahead of writes
+  const int n = b0 - a0, keep = K - 1;
+  float* tl = tail + (size_t)slot * (keep > 0 ? keep : 1) * C;
+  const float xb = x_bias[c];
+  for (int i = 0; i < keep; ++i) {
+    const int src = n + i;                     // place in the joined sequence of keep + n inputs
+    tl[(size_t)i * C + c] = src < keep ? tl[(size_t)src * C + c] : x[(size_t)(a0 + src - keep) * ldx + c] + xb;
+  }
+}
+
+MIE_EXPORT const char* recurrence_last_error() { return g_mie_error; }
+
+// x points at the first of the C input columns (rows ldx floats apart); taps [C, K]; tail [slots, max(1, K - 1), C].
+MIE_EXPORT int mie_causal_conv(const float* x, long ldx, const float* in_bias, const float* taps, const float* conv_bias,
+                               const float* tail, const int* token_row, const int* row_start, const int* slots, float* u,
+                               int tokens, int C, int K, hipStream_t s) {
+  if (tokens <= 0) return 0;
+  if (C <= 0 || K <= 0 || ldx < C) MIE_FAIL("causal_conv: %d channels, %d taps, row stride %ld", C, K, ldx);
+  if (!x || !in_bias || !taps || !conv_bias || !tail || !token_row || !row_start || !slots || !u) MIE_FAIL("causal_conv: operands");
+  const int by = (C + 255) / 256;
+  hipLaunchKernelGGL(causal_conv_kernel, dim3(tokens, by > 64 ? 64 : by), dim3(256), 0, s, x, ldx, in_bias, taps, conv_bias, tail,
+                     token_row, row_start, slots, u, C, K);
+  MIE_CHECK_LAUNCH("causal_conv");
+  return 0;
+}
+
+// u [tokens, C], gates [tokens, 2 C] contiguous; y, x point at their first column; out [tokens, C] of out_dtype.
+MIE_EXPORT int mie_rglru_scan(const float* u, const float* gates, const float* lam, const float* y, long ldy,
+                              const float* y_bias, const float* x, long ldx, const float* x_bias, float* state, float* tail,
+                              const int* row_start, const int* slots, void* out, int out_dtype, int rows, int C, int K,
+                              float decay_scale, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (C <= 0 || K <= 0 || ldy < C || ldx < C) MIE_FAIL("rglru_scan: %d channels, %d taps, row strides %ld, %ld", C, K, ldy, ldx);
+  if (!u || !gates || !lam || !y || !y_bias || !x || !x_bias || !state || !tail || !row_start || !slots || !out)
+    MIE_FAIL("rglru_scan: operands");
+  dim3 grid(rows, (C + 255) / 256);
+  if (out_dtype == MIE_F32)
+    hipLaunchKernelGGL(rglru_scan_kernel<float>, grid, dim3(256), 0, s, u, gates, lam, y, ldy, y_bias, x, ldx, x_bias, state, tail,
+                       row_start, slots, (float*)out, C, K, decay_scale);
+  else if (out_dtype == MIE_BF16)
+    hipLaunchKernelGGL(rglru_scan_kernel<bf16>, grid, dim3(256), 0, s, u, gates, lam, y, ldy, y_bias, x, ldx, x_bias, state, tail,
+                       row_start, slots, (bf16*)out, C, K, decay_scale);
+  else
+    MIE_FAIL("rglru_scan: output dtype code %d", out_dtype);
+  MIE_CHECK_LAUNCH("rglru_scan");
+  return 0;
+}

@@ -123,8 +123,8 @@ class KernelBackend:
         [c | zeros] (P = the cache's padded size >= kv_rank + rot_dim)."""
         raise NotImplementedError
 
-    def latent_query(self, q, w_uk, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim):
-        """q [T, H (dim + rot_dim)]; w_uk [H dim, kv_rank].  Per head h: [q_h[:dim] W_uk,h | turned q_h[dim:] | zeros]
+    def latent_query(self, q, w_uk_t, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim):
+        """q [T, H (dim + rot_dim)]; w_uk_t [kv_rank, H dim], the transpose of W_uk [H dim, kv_rank].  Per head h: [q_h[:dim] W_uk,h | turned q_h[dim:] | zeros]
         -> [T, H padded_dim] in the activation dtype: the query against a cached latent, since
         q_h[:dim] . (W_uk,h c) = (q_h[:dim] W_uk,h) . c."""
         raise NotImplementedError
@@ -149,11 +149,11 @@ class KernelBackend:
         32-bit arithmetic throughout."""
         raise NotImplementedError
 
-    def rglru_scan(self, u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, step, decay_scale=8.0):
+    def rglru_scan(self, u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, step, taps, decay_scale=8.0):
         """Per row and channel, tokens in order: r, i = sigmoid of gates[t, c], gates[t, C + c];
         a = exp(-decay_scale * r * softplus(lam[c])); S = a S + sqrt(1 - a^2) * i * u[t, c] from the row's slot of
         ``state`` [slots, C] float32, left there afterwards; out[t, c] = S * gelu_tanh(y[t, y_col + c] + y_bias[c]).
-        Also shifts the row's inputs x[t, x_col + c] + x_bias[c] into ``tail`` [slots, K - 1, C].  All float32;
+        Also shifts the row's inputs x[t, x_col + c] + x_bias[c] into ``tail`` [slots, max(1, taps - 1), C].  All float32;
         -> [T, C] in the activation dtype."""
         raise NotImplementedError
 

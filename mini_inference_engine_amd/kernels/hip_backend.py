@@ -146,7 +146,7 @@ class HipBackend(KernelBackend):
         return out
 
     # ----------------------------------------------------------------- ops
-    def embedding(self, ids, table, taken_from=None, earlier_tokens=None):
+    def embedding(self, ids, table, taken_from=None, earlier_tokens=None, scale=1.0):
         self._on_device(ids, table, taken_from, earlier_tokens)
         if ids.dtype != torch.int32 or ids.dim() != 1 or not ids.is_contiguous():
             raise ValueError("embedding: ids must be contiguous int32 [T]")
@@ -160,7 +160,7 @@ class HipBackend(KernelBackend):
         out = torch.empty((T, W), dtype=torch.float32, device=table.device)
         lib = self.lib("embed_norm")
         library.check(lib, lib.mie_embedding(_ptr(ids), _ptr(table), _code(table.dtype), _ptr(out), T, W, V,
-                                             _ptr(taken_from), _ptr(earlier_tokens), self._stream()))
+                                             _ptr(taken_from), _ptr(earlier_tokens), float(scale), self._stream()))
         return out
 
     def add_rmsnorm(self, x, residual, weight, eps, out_dtype=None, rows=None):
@@ -386,6 +386,263 @@ class HipBackend(KernelBackend):
             self._skinny(x, w_gate_up, self.EPI_SWIGLU, out, intermediate)
             return out
         return self.silu_mul(self.linear(x, w_gate_up), intermediate)
+
+    ACT_CODES = {"none": 0, "silu": 1, "gelu_tanh": 2, "relu2": 3}
+
+    def linear_act_mul(self, x, w_gate_up, intermediate, activation="silu"):
+        if activation == "silu":
+            return self.linear_silu_mul(x, w_gate_up, intermediate)
+        if activation not in self.ACT_CODES:
+            raise ValueError(f"linear_act_mul: activation {activation!r}")
+        if w_gate_up.shape[0] != 2 * intermediate or x.shape[1] != w_gate_up.shape[1]:
+            raise ValueError(f"linear_act_mul: x {tuple(x.shape)}, w {tuple(w_gate_up.shape)}, intermediate {intermediate}")
+        gu = self.linear(x, w_gate_up)
+        out = torch.empty((gu.shape[0], intermediate), dtype=gu.dtype, device=gu.device)
+        lib = self.lib("gemm")
+        library.check(lib, lib.mie_act_mul(_ptr(gu), gu.stride(0), _ptr(out), out.stride(0), _code(gu.dtype), gu.shape[0],
+                                           intermediate, self.ACT_CODES[activation], self._stream()))
+        return out
+
+    def scale_(self, t, factor):
+        self._on_device(t)
+        if t.dtype != torch.float32 or not t.is_contiguous():
+            raise ValueError("scale_: a contiguous float32 tensor")
+        lib = self.lib("embed_norm")
+        library.check(lib, lib.mie_scale(_ptr(t), t.numel(), float(factor), self._stream()))
+        return t
+
+    def branch_norm_add(self, y, stream, weight, eps):
+        self._on_device(y, stream, weight)
+        if stream.dtype != torch.float32 or stream.dim() != 2 or not stream.is_contiguous():
+            raise ValueError("branch_norm_add: the stream must be contiguous float32 [T, width]")
+        T, W = stream.shape
+        if y is not None:
+            if tuple(y.shape) != (T, W) or not y.is_contiguous():
+                raise ValueError(f"branch_norm_add: y {tuple(y.shape)} does not match the stream {(T, W)}")
+            if weight is None or tuple(weight.shape) != (W,) or not weight.is_contiguous():
+                raise ValueError(f"branch_norm_add: a contiguous weight of {W}")
+        copy = None if self.act_dtype == torch.float32 else torch.empty((T, W), dtype=self.act_dtype, device=stream.device)
+        if y is not None or copy is not None:
+            lib = self.lib("embed_norm")
+            library.check(lib, lib.mie_branch_norm_add(
+                _ptr(y), _code(y.dtype) if y is not None else F32, _ptr(stream), _ptr(weight),
+                _code(weight.dtype) if weight is not None else F32, _ptr(copy), _code(copy.dtype) if copy is not None else F32,
+                T, W, float(eps), self._stream()))
+        return stream if copy is None else copy
+
+    @staticmethod
+    def _f32_columns(x, col, n, what):
+        if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1 or col < 0 or col + n > x.shape[1]:
+            raise ValueError(f"{what}: columns {col} .. {col + n} of a float32 matrix with unit inner stride, got "
+                             f"{tuple(x.shape)} {x.dtype}")
+        return c_void_p(x.data_ptr() + 4 * col)
+
+    @staticmethod
+    def _f32_vector(t, n, what):
+        if t is None or t.dtype != torch.float32 or t.numel() != n or not t.is_contiguous():
+            raise ValueError(f"{what}: {n} contiguous float32 numbers expected")
+        return _ptr(t)
+
+    def rmsnorm_columns(self, x, col, n, weight, eps):
+        self._on_device(x, weight)
+        xp = self._f32_columns(x, col, n, "rmsnorm_columns")
+        if tuple(weight.shape) != (n,) or not weight.is_contiguous():
+            raise ValueError(f"rmsnorm_columns: weight {tuple(weight.shape)} for {n} columns")
+        out = torch.empty((x.shape[0], n), dtype=self.act_dtype, device=x.device)
+        lib = self.lib("embed_norm")
+        library.check(lib, lib.mie_rmsnorm_columns(xp, x.stride(0), _ptr(weight), _code(weight.dtype), _ptr(out),
+                                                   _code(out.dtype), x.shape[0], n, float(eps), self._stream()))
+        return out
+
+    # ---- many small products in one launch
+    def _grouped(self, A, lda, a_group, a_mod, W, ldw, w_group, C, ldc, c_group, M, N, K, G, bias=None, gate=None, ldg=0,
+                 offs=None, gather=None, gather_div=1, act="none"):
+        lib = self.lib("grouped_gemm")
+        library.check(lib, lib.mie_grouped_linear(
+            _ptr(A), _code(A.dtype), lda, a_group, a_mod, _ptr(W), _code(W.dtype), ldw, w_group, _ptr(C), _code(C.dtype), ldc,
+            c_group, _ptr(bias), gate, ldg, _ptr(offs), _ptr(gather), gather_div, M, N, K, G, self.ACT_CODES[act],
+            self._stream()))
+
+    def grouped_linear(self, x, w, bias=None, x_groups=None):
+        self._on_device(x, w, bias)
+        _rows_ok(x, "grouped_linear: x")
+        if w.dim() != 3 or not w.is_contiguous():
+            raise ValueError("grouped_linear: w must be contiguous [groups, out, in]")
+        G, N, K = w.shape
+        gx = int(x_groups or G)
+        if x.shape[1] != gx * K:
+            raise ValueError(f"grouped_linear: x {tuple(x.shape)} for {gx} blocks of {K}")
+        if bias is not None:
+            self._f32_vector(bias, G * N, "grouped_linear: bias")
+        out = torch.empty((x.shape[0], G * N), dtype=torch.float32, device=x.device)
+        self._grouped(x, x.stride(0), K, gx, w, K, N * K, out, G * N, N, x.shape[0], N, K, G, bias=bias)
+        return out
+
+    # ---- attention through a cached latent
+    def _check_latent_cache(self, what, k_cache, v_cache, kv_rank, rot_dim):
+        pages, one, page, P = k_cache.shape
+        if one != 1 or tuple(v_cache.shape) != (pages, 1, P, page) or P < kv_rank + rot_dim:
+            raise ValueError(f"{what}: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} for a latent of {kv_rank} + {rot_dim}")
+        if k_cache.dtype != v_cache.dtype or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+            raise ValueError(f"{what}: caches must be contiguous and of one dtype")
+        return page, P
+
+    def latent_kv_store(self, sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache,
+                        slot_mapping):
+        self._on_device(sums, norm_weight, positions, inv_freq, k_cache, v_cache, slot_mapping)
+        sp = self._f32_columns(sums, col, kv_rank + rot_dim, "latent_kv_store")
+        T = sums.shape[0]
+        page, P = self._check_latent_cache("latent_kv_store", k_cache, v_cache, kv_rank, rot_dim)
+        if tuple(norm_weight.shape) != (kv_rank,) or not norm_weight.is_contiguous():
+            raise ValueError(f"latent_kv_store: norm weight {tuple(norm_weight.shape)} for a latent of {kv_rank}")
+        n_freq = inv_freq.numel()
+        self._f32_vector(inv_freq, n_freq, "latent_kv_store: inv_freq")
+        for name, t in (("positions", positions), ("slot_mapping", slot_mapping)):
+            if t.dtype != torch.int32 or t.shape[0] != T or not t.is_contiguous():
+                raise ValueError(f"latent_kv_store: {name} must be contiguous int32 [{T}]")
+        lib = self.lib("latent_attention")
+        library.check(lib, lib.mie_latent_kv_store(
+            sp, sums.stride(0), _ptr(norm_weight), _code(norm_weight.dtype), float(eps), _ptr(positions), _ptr(inv_freq), n_freq,
+            _ptr(k_cache), _ptr(v_cache), _code(k_cache.dtype), _ptr(slot_mapping), T, kv_rank, rot_dim, P, page, self._stream()))
+
+    def latent_query(self, q, w_uk_t, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim):
+        self._on_device(q, w_uk_t, positions, inv_freq)
+        _rows_ok(q, "latent_query: q")
+        H, P, T = num_heads, padded_dim, q.shape[0]
+        if q.shape[1] != H * (dim + rot_dim) or tuple(w_uk_t.shape) != (kv_rank, H * dim) or not w_uk_t.is_contiguous():
+            raise ValueError(f"latent_query: q {tuple(q.shape)}, w {tuple(w_uk_t.shape)} for {H} heads of {dim} + {rot_dim}, "
+                             f"latent {kv_rank}")
+        if P < kv_rank + rot_dim or positions.dtype != torch.int32 or positions.shape[0] != T or not positions.is_contiguous():
+            raise ValueError("latent_query: padded size or positions")
+        n_freq = inv_freq.numel()
+        self._f32_vector(inv_freq, n_freq, "latent_query: inv_freq")
+        out = torch.empty((T, H * P), dtype=q.dtype, device=q.device)
+        # head h: q[:, h (dim + rot_dim) : + dim] times the columns h dim .. of the transposed W_uk -> out[:, h P : + kv_rank]
+        self._grouped(q, q.stride(0), dim + rot_dim, H, w_uk_t, H * dim, dim, out, H * P, P, T, kv_rank, dim, H)
+        lib = self.lib("latent_attention")
+        library.check(lib, lib.mie_latent_query_rotate(_ptr(q), q.stride(0), _ptr(out), _code(q.dtype), _ptr(positions),
+                                                       _ptr(inv_freq), n_freq, T, H, dim, rot_dim, kv_rank, P, self._stream()))
+        return out
+
+    def latent_value_gate(self, o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim):
+        self._on_device(o, w_uv, gate)
+        H, P, T = num_heads, padded_dim, o.shape[0]
+        if tuple(o.shape) != (T, H * P) or not o.is_contiguous() or tuple(w_uv.shape) != (H * vdim, kv_rank) or not w_uv.is_contiguous():
+            raise ValueError(f"latent_value_gate: o {tuple(o.shape)}, w {tuple(w_uv.shape)} for {H} heads of {vdim}, latent {kv_rank}")
+        gp, ldg = None, 0
+        if gate is not None:
+            gp, ldg = self._f32_columns(gate, gate_col, H * vdim, "latent_value_gate: gate"), gate.stride(0)
+            if gate.shape[0] != T:
+                raise ValueError("latent_value_gate: one gate row a token")
+        out = torch.empty((T, H * vdim), dtype=o.dtype, device=o.device)
+        self._grouped(o, H * P, P, H, w_uv, kv_rank, vdim * kv_rank, out, H * vdim, vdim, T, vdim, kv_rank, H, gate=gp, ldg=ldg)
+        return out
+
+    # ---- gated linear recurrence
+    def _check_rows(self, what, step, T):
+        for name, t, n in (("token_row", step.token_row, T), ("row_start", step.row_start, step.num_rows + 1),
+                           ("state_slots", step.state_slots, step.num_rows)):
+            if t is None or t.dtype != torch.int32 or t.shape[0] < n or not t.is_contiguous():
+                raise ValueError(f"{what}: {name} must be contiguous int32 [{n}]")
+        if step.num_tokens != T:
+            raise ValueError(f"{what}: {T} tokens for a step of {step.num_tokens}")
+
+    def causal_conv(self, x, col, channels, in_bias, taps, conv_bias, tail, step):
+        self._on_device(x, in_bias, taps, conv_bias, tail)
+        C, T = channels, x.shape[0]
+        xp = self._f32_columns(x, col, C, "causal_conv")
+        if taps.dim() != 2 or taps.shape[0] != C:
+            raise ValueError(f"causal_conv: taps {tuple(taps.shape)} for {C} channels")
+        K = taps.shape[1]
+        self._f32_vector(taps, C * K, "causal_conv: taps")
+        self._f32_vector(in_bias, C, "causal_conv: input bias")
+        self._f32_vector(conv_bias, C, "causal_conv: bias")
+        if tail.dtype != torch.float32 or tuple(tail.shape[1:]) != (max(1, K - 1), C) or not tail.is_contiguous():
+            raise ValueError(f"causal_conv: tail {tuple(tail.shape)} for {K} taps of {C} channels")
+        self._check_rows("causal_conv", step, T)
+        if int(step.host["state_slots"].max()) >= tail.shape[0]:
+            raise ValueError("causal_conv: a state slot beyond the tail's slots")
+        u = torch.empty((T, C), dtype=torch.float32, device=x.device)
+        lib = self.lib("recurrence")
+        library.check(lib, lib.mie_causal_conv(xp, x.stride(0), _ptr(in_bias), _ptr(taps), _ptr(conv_bias), _ptr(tail),
+                                               _ptr(step.token_row), _ptr(step.row_start), _ptr(step.state_slots), _ptr(u),
+                                               T, C, K, self._stream()))
+        return u
+
+    def rglru_scan(self, u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, step, taps, decay_scale=8.0):
+        self._on_device(u, gates, lam, y, y_bias, x, x_bias, state, tail)
+        T, C = u.shape
+        if u.dtype != torch.float32 or not u.is_contiguous() or gates.dtype != torch.float32 or tuple(gates.shape) != (T, 2 * C) \
+                or not gates.is_contiguous():
+            raise ValueError(f"rglru_scan: u {tuple(u.shape)} and gates {tuple(gates.shape)} must be contiguous float32 [T, C], [T, 2 C]")
+        yp = self._f32_columns(y, y_col, C, "rglru_scan: y")
+        xp = self._f32_columns(x, x_col, C, "rglru_scan: x")
+        if y.shape[0] != T or x.shape[0] != T:
+            raise ValueError("rglru_scan: one row of y and x a token")
+        for name, t in (("lam", lam), ("y_bias", y_bias), ("x_bias", x_bias)):
+            self._f32_vector(t, C, f"rglru_scan: {name}")
+        K = int(taps)
+        if state.dtype != torch.float32 or state.dim() != 2 or state.shape[1] != C or not state.is_contiguous() \
+                or tail.dtype != torch.float32 or tuple(tail.shape) != (state.shape[0], max(1, K - 1), C) \
+                or not tail.is_contiguous():
+            raise ValueError(f"rglru_scan: state {tuple(state.shape)}, tail {tuple(tail.shape)} for {C} channels")
+        self._check_rows("rglru_scan", step, T)
+        if int(step.host["state_slots"].max()) >= state.shape[0]:
+            raise ValueError("rglru_scan: a state slot beyond the state's slots")
+        out = torch.empty((T, C), dtype=self.act_dtype, device=u.device)
+        lib = self.lib("recurrence")
+        library.check(lib, lib.mie_rglru_scan(_ptr(u), _ptr(gates), _ptr(lam), yp, y.stride(0), _ptr(y_bias), xp, x.stride(0),
+                                              _ptr(x_bias), _ptr(state), _ptr(tail), _ptr(step.row_start), _ptr(step.state_slots),
+                                              _ptr(out), _code(out.dtype), step.num_rows, C, K, float(decay_scale), self._stream()))
+        return out
+
+    # ---- routed experts
+    def route_topk(self, logits, bias, top):
+        self._on_device(logits, bias)
+        if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
+            raise ValueError("route_topk: logits must be float32 [T, experts] with unit inner stride")
+        T, E = logits.shape
+        if bias is not None:
+            self._f32_vector(bias, E, "route_topk: bias")
+        if not 1 <= top <= min(E, 16):
+            raise ValueError(f"route_topk: top {top} of {E} experts (at most 16)")
+        experts = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+        shares = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+        lib = self.lib("grouped_gemm")
+        library.check(lib, lib.mie_route_topk(_ptr(logits), logits.stride(0), _ptr(bias), _ptr(experts), _ptr(shares), T, E, top,
+                                              self._stream()))
+        return experts, shares
+
+    def routed_experts(self, x, experts, shares, w_up, w_down, activation="relu2"):
+        self._on_device(x, experts, shares, w_up, w_down)
+        _rows_ok(x, "routed_experts: x")
+        T, W = x.shape
+        if w_up.dim() != 3 or w_down.dim() != 3 or not (w_up.is_contiguous() and w_down.is_contiguous()):
+            raise ValueError("routed_experts: contiguous [experts, ff, width] and [experts, width, ff]")
+        E, ff, _ = w_up.shape
+        if w_up.shape[2] != W or tuple(w_down.shape) != (E, W, ff):
+            raise ValueError(f"routed_experts: w_up {tuple(w_up.shape)}, w_down {tuple(w_down.shape)} for width {W}")
+        top = experts.shape[1]
+        if experts.dtype != torch.int32 or tuple(experts.shape) != (T, top) or not experts.is_contiguous() \
+                or shares.dtype != torch.float32 or tuple(shares.shape) != (T, top) or not shares.is_contiguous():
+            raise ValueError("routed_experts: experts int32 [T, top] and shares float32 [T, top], contiguous")
+        if activation not in self.ACT_CODES:
+            raise ValueError(f"routed_experts: activation {activation!r}")
+        n = T * top
+        dev = x.device
+        offs = torch.empty(E + 1, dtype=torch.int32, device=dev)
+        order = torch.empty(n, dtype=torch.int32, device=dev)
+        place = torch.empty(n, dtype=torch.int32, device=dev)
+        lib = self.lib("grouped_gemm")
+        library.check(lib, lib.mie_moe_align(_ptr(experts), n, E, _ptr(offs), _ptr(order), _ptr(place), self._stream()))
+        hidden = torch.empty((n, ff), dtype=self.act_dtype, device=dev)
+        self._grouped(x, x.stride(0), 0, 1, w_up, W, ff * W, hidden, ff, 0, n, ff, W, E, offs=offs, gather=order, gather_div=top,
+                      act=activation)
+        y = torch.empty((n, W), dtype=torch.float32, device=dev)
+        self._grouped(hidden, ff, 0, 1, w_down, ff, W * ff, y, W, 0, n, W, ff, E, offs=offs)
+        out = torch.empty((T, W), dtype=torch.float32, device=dev)
+        library.check(lib, lib.mie_moe_combine(_ptr(y), _ptr(place), _ptr(shares), _ptr(out), T, W, top, self._stream()))
+        return out
 
     def linear_rotary_kv_store(self, x, w_qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
                                k_cache, v_cache, slot_mapping, for_attention: bool = False):

@@ -10,8 +10,11 @@ P, I, L, F = c_void_p, c_int, c_long, c_float
 _head_variants = [(f"-DHEAD_DIM={d}",) for d in HEAD_DIMS]
 
 register_kernel_module("embed_norm", {
-    "mie_embedding": [P, P, I, P, I, I, I, P, P, P],
+    "mie_embedding": [P, P, I, P, I, I, I, P, P, F, P],
     "mie_add_rmsnorm": [P, I, P, P, I, P, I, P, I, I, F, P],
+    "mie_branch_norm_add": [P, I, P, P, I, P, I, I, I, F, P],
+    "mie_rmsnorm_columns": [P, L, P, I, P, I, I, I, F, P],
+    "mie_scale": [P, L, F, P],
 })
 register_kernel_module("rope_kv", {
     "mie_rotary_kv_store": [P, I, L, P, P, P, I, I, I, I, P, P, P, I, I, P],
@@ -20,6 +23,21 @@ register_kernel_module("rope_kv", {
 register_kernel_module("gemm", {
     "mie_gemm_nt": [P, I, L, P, I, L, P, I, L, P, I, I, I, P],
     "mie_silu_mul": [P, L, P, L, I, I, I, P],
+    "mie_act_mul": [P, L, P, L, I, I, I, I, P],
+})
+register_kernel_module("grouped_gemm", {
+    "mie_grouped_linear": [P, I, L, L, I, P, I, L, L, P, I, L, L, P, P, L, P, P, I, I, I, I, I, I, P],
+    "mie_route_topk": [P, L, P, P, P, I, I, I, P],
+    "mie_moe_align": [P, I, I, P, P, P, P],
+    "mie_moe_combine": [P, P, P, P, I, I, I, P],
+})
+register_kernel_module("latent_attention", {
+    "mie_latent_kv_store": [P, L, P, I, F, P, P, I, P, P, I, P, I, I, I, I, I, P],
+    "mie_latent_query_rotate": [P, L, P, I, P, P, I, I, I, I, I, I, I, P],
+})
+register_kernel_module("recurrence", {
+    "mie_causal_conv": [P, L, P, P, P, P, P, P, P, P, I, I, I, P],
+    "mie_rglru_scan": [P, P, P, P, L, P, P, L, P, P, P, P, P, P, I, I, I, I, F, P],
 })
 register_kernel_module("attention", {
     "mie_paged_attention": [P, L, P, P, P, I, P, I, P, P, I, I, I, I, I, F, I, P],

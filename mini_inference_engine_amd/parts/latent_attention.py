@@ -18,7 +18,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 
-from .base import CacheRequirement, Mixer, ParamSpec, register_mixer
+from .base import CacheRequirement, Mixer, ParamSpec, Source, register_mixer
 
 DEFAULT_NAMES = dict(dq="dq", dq_norm="dq.norm", uq="uq", dkv="dkv", dkv_norm="dkv.norm", uk="uk", uv="uv", g="g", o="o")
 
@@ -82,7 +82,10 @@ class LatentAttention(Mixer):
         specs = [ParamSpec.stacked("w_down", down),
                  ParamSpec.single("dq_norm", name("dq_norm"), (self.q_rank,), init="scale"),
                  ParamSpec.single("w_uq", name("uq"), (H * (self.dim + self.rot_dim), self.q_rank)),
-                 ParamSpec.single("w_uk", name("uk"), (H * self.dim, self.kv_rank)),
+                 # W_uk is folded into the queries, head by head: kept transposed, [kv_rank, H dim]
+                 ParamSpec("w_uk_t", (self.kv_rank, H * self.dim),
+                           (Source(name("uk"), (self.kv_rank, H * self.dim), 0, stored_shape=(H * self.dim, self.kv_rank),
+                                   transform="transpose"),)),
                  ParamSpec.single("w_uv", name("uv"), (H * self.vdim, self.kv_rank)),
                  ParamSpec.single("w_o", name("o"), (w, H * self.vdim))]
         if self.has_kv:
@@ -110,7 +113,7 @@ class LatentAttention(Mixer):
             col += self.kv_rank + self.rot_dim
         cq = ops.rmsnorm_columns(sums, 0, self.q_rank, self.dq_norm, self.eps)
         q = ops.linear(cq, self.w_uq)
-        q = ops.latent_query(q, self.w_uk, self.num_heads, self.dim, self.rot_dim, self.kv_rank, step.positions, inv_freq,
+        q = ops.latent_query(q, self.w_uk_t, self.num_heads, self.dim, self.rot_dim, self.kv_rank, step.positions, inv_freq,
                              self.padded_dim)
         o = ops.paged_attention(q, self.num_heads, 1, self.padded_dim, cache.k, cache.v, group, step, self.scale, None)
         heads = ops.latent_value_gate(o, self.w_uv, sums if self.gated else None, col, self.num_heads, self.vdim,

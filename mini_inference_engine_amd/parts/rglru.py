@@ -66,6 +66,11 @@ class RGLRU(Mixer):
     def cache_requirement(self):
         return RecurrentState(self.channels, self.taps)
 
+    def prepare(self, device, dtype):
+        # the recurrence, its gates' biases and the convolution are 32-bit whatever the checkpoint stores
+        for attr in ("b_in", "conv", "conv_bias", "b_gates", "lam"):
+            setattr(self, attr, getattr(self, attr).float().contiguous())
+
     def forward(self, x, step, cache, add_to=None):
         import torch
         ops, C = self.ops, self.channels
@@ -74,5 +79,5 @@ class RGLRU(Mixer):
         b_y, b_x = self.b_in[:C], self.b_in[C:]
         u = ops.causal_conv(sums, C, C, b_x, self.conv, self.conv_bias, tail, step)
         gates = ops.grouped_linear(u, self.w_gates, self.b_gates, x_groups=self.blocks)
-        out = ops.rglru_scan(u, gates, self.lam, sums, 0, b_y, sums, C, b_x, state, tail, step, self.decay_scale)
+        out = ops.rglru_scan(u, gates, self.lam, sums, 0, b_y, sums, C, b_x, state, tail, step, self.taps, self.decay_scale)
         return ops.linear(out, self.w_o, out_dtype=torch.float32)

@@ -34,6 +34,10 @@ class RoutedExperts(FeedForward):
             specs.append(ParamSpec.single("b_router", f"{p}.{n['router_bias']}", (E,), init="zeros"))
         return specs
 
+    def prepare(self, device, dtype):
+        if self.router_bias:
+            self.b_router = self.b_router.float().contiguous()      # router logits are 32-bit
+
     def forward(self, x, step, add_to=None):
         import torch
         ops, E = self.ops, self.num_experts

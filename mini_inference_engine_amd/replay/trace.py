@@ -100,8 +100,10 @@ def main(argv=None) -> int:
     # request that may be live keeps a count that was not rounded from running out (a request wastes less than a
     # page), + the scratch page
     pages = -(-args.max_tokens // page) + live + 1
+    # no request can be longer than the pool holds (a model without a longest position of its own would otherwise
+    # size every row's block table for a position nobody reaches)
     runner = ModelRunner(args.model, dtype=args.dtype, device=args.device, page_size=page, num_pages=pages,
-                         max_step_tokens=max(64, args.max_tokens), max_rows=live)
+                         max_step_tokens=max(64, args.max_tokens), max_rows=live, max_model_len=(pages - 1) * page)
     if args.hip_graphs:
         runner.capture_decode_graphs(tuple(b for b in (1, 2, 4, 8, 16, 32, 64) if b < 2 * live))
 

@@ -66,11 +66,11 @@ def ref_latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions
     v_cache[page, 0, :kv_rank, off] = c.to(v_cache.dtype)
 
 
-def ref_latent_query(q, w_uk, H, dim, rot_dim, kv_rank, positions, inv_freq, padded, out_dtype):
+def ref_latent_query(q, w_uk_t, H, dim, rot_dim, kv_rank, positions, inv_freq, padded, out_dtype):
     T = q.shape[0]
     qh = q.double().view(T, H, dim + rot_dim)
     out = torch.zeros(T, H, padded, dtype=torch.float64, device=q.device)
-    out[..., :kv_rank] = torch.einsum("thd,hdr->thr", qh[..., :dim], w_uk.double().view(H, dim, kv_rank))
+    out[..., :kv_rank] = torch.einsum("thd,rhd->thr", qh[..., :dim], w_uk_t.double().view(kv_rank, H, dim))
     out[..., kv_rank:kv_rank + rot_dim] = ref_turn_pairs(qh[..., dim:], positions, inv_freq)
     return out.view(T, H * padded).to(out_dtype)
 
@@ -107,9 +107,9 @@ def ref_grouped_linear(x, w, bias, x_groups):
     return y.reshape(x.shape[0], G * n_out).float()
 
 
-def ref_rglru_scan(u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, row_start, slots, decay_scale, out_dtype):
+def ref_rglru_scan(u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, row_start, slots, taps, decay_scale, out_dtype):
     C = u.shape[1]
-    K1 = tail.shape[1]
+    K1 = taps - 1
     out = torch.empty(u.shape[0], C, dtype=torch.float64, device=u.device)
     sp = torch.nn.functional.softplus(lam.double())
     for r in range(len(slots)):
@@ -121,8 +121,9 @@ def ref_rglru_scan(u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tai
             S = a * S + torch.sqrt(1.0 - a * a) * ig * u[t].double()
             out[t] = S * ref_act(y[t, y_col:y_col + C].double() + y_bias.double(), "gelu_tanh")
         state[slot] = S.float()
-        inp = torch.cat([tail[slot].double(), x[a0:b0, x_col:x_col + C].double() + x_bias.double()])
-        tail[slot] = inp[-K1:].float()
+        if K1:
+            inp = torch.cat([tail[slot][:K1].double(), x[a0:b0, x_col:x_col + C].double() + x_bias.double()])
+            tail[slot][:K1] = inp[-K1:].float()
     return out.to(out_dtype)
 
 
@@ -283,8 +284,8 @@ class TorchBackend(KernelBackend):
         self._count("latent_kv_store")
         ref_latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache, slot_mapping)
 
-    def latent_query(self, q, w_uk, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim):
-        return ref_latent_query(q, w_uk, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim, self.act_dtype)
+    def latent_query(self, q, w_uk_t, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim):
+        return ref_latent_query(q, w_uk_t, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim, self.act_dtype)
 
     def latent_value_gate(self, o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim):
         return ref_latent_value_gate(o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim, self.act_dtype)
@@ -296,10 +297,10 @@ class TorchBackend(KernelBackend):
     def grouped_linear(self, x, w, bias=None, x_groups=None):
         return ref_grouped_linear(x, w, bias, x_groups)
 
-    def rglru_scan(self, u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, step, decay_scale=8.0):
+    def rglru_scan(self, u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, step, taps, decay_scale=8.0):
         self._count("rglru_scan")
         return ref_rglru_scan(u, gates, lam, y, y_col, y_bias, x, x_col, x_bias, state, tail, step.host["row_start"],
-                              step.host["state_slots"], decay_scale, self.act_dtype)
+                              step.host["state_slots"], taps, decay_scale, self.act_dtype)
 
     def route_topk(self, logits, bias, top):
         return ref_route_topk(logits, bias, top)
