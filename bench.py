@@ -3,6 +3,8 @@ Llama-2-7B or Llama-3-8B), random weights.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--shape tinyllama] [--context N] [--layers L]
     python bench.py --kernels [--shape ...] [--batch 8] [--context N]     each dominant kernel alone
+    python bench.py --design zifelorn [--design-sizes 1024,2048] [--layers R] [--batch 8] [--context 1024]
+                                                 Zifelorn beside Llama at equal layer sizes (R runs of four layers)
 
 A step is one decode step of the engine (schedule, batch, captured forward, sampling,
 bookkeeping: LLMEngine.step, the call a user's loop makes; it starts a step and reads the tokens
@@ -128,7 +130,7 @@ def prompts_of(n: int, length: int, vocab: int, seed: int):
     return [torch.randint(0, vocab, (length,), generator=g).tolist() for _ in range(n)]
 
 
-def measure_decode(eng, batch: int, context: int, steps: int, warmup: int, seed: int):
+def measure_decode(eng, batch: int, context: int, steps: int, warmup: int, seed: int, vocab: int | None = None):
     """Median-free, as the contract asks: exactly ``steps`` steps between two synchronisations."""
     import torch
     from mini_inference_engine_amd import SamplingParams
@@ -138,7 +140,7 @@ def measure_decode(eng, batch: int, context: int, steps: int, warmup: int, seed:
     slack = -(-batch * context // budget) + 2
     prompt_len = context - (steps + warmup + slack + 3)
     assert prompt_len >= 1, "context too short for that many steps"
-    for p in prompts_of(batch, prompt_len, eng.model_cfg.vocab_size, seed):
+    for p in prompts_of(batch, prompt_len, vocab or eng.model_cfg.vocab_size, seed):
         eng.add_request(p, SamplingParams(max_tokens=steps + warmup + slack + 2, ignore_eos=True))
     while eng.scheduler.waiting or any(s.num_new_tokens > 1 for s in eng.scheduler.running):
         eng.step()
@@ -159,12 +161,12 @@ def measure_decode(eng, batch: int, context: int, steps: int, warmup: int, seed:
     return dt, captured, mid_context
 
 
-def measure_prefill(eng, tokens: int, seed: int):
+def measure_prefill(eng, tokens: int, seed: int, vocab: int | None = None):
     import torch
     from mini_inference_engine_amd import SamplingParams
     times = []
     for rep in range(6):                      # the first run loads libraries and picks GEMM kernels
-        p = prompts_of(1, tokens, eng.model_cfg.vocab_size, seed + rep)[0]
+        p = prompts_of(1, tokens, vocab or eng.model_cfg.vocab_size, seed + rep)[0]
         eng.add_request(p, SamplingParams(max_tokens=1, ignore_eos=True))
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -425,8 +427,68 @@ def measure_kernels(cfg, args) -> int:
     return 0
 
 
+# ---------------------------------------------------------------------------- two designs at equal sizes
+# Zifelorn layer sizes that resemble a real model's, and the Llama configuration of the same width, head count,
+# feed-forward size, vocabulary and layer count beside each.  A Zifelorn run of four layers is latent attention +
+# dense, latent attention + experts, recurrence + dense, latent attention on the second layer's cache + experts.
+DESIGN_SIZES = {
+    "1024": dict(vocab=32000, width=1024, heads=8, dim=64, rot_dim=32, vdim=64, kv_rank=128, q_rank=384, channels=1280,
+                 blocks=5, ff=2816, experts=8, top=2, expert_ff=704),
+    "2048": dict(vocab=32000, width=2048, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=192, q_rank=768, channels=2560,
+                 blocks=10, ff=5632, experts=16, top=2, expert_ff=1408),
+}
+
+
+def design_configs(size: str, repeats: int):
+    from mini_inference_engine_amd.config import LlamaConfig, ZifelornConfig
+    from mini_inference_engine_amd.models.zifelorn import _shape
+    z = DESIGN_SIZES[size]
+    zcfg = ZifelornConfig.from_dict(_shape(repeats=repeats, **z))
+    lcfg = LlamaConfig.from_dict(dict(
+        vocab_size=z["vocab"], hidden_size=z["width"], intermediate_size=z["ff"], num_hidden_layers=4 * repeats,
+        num_attention_heads=z["heads"], num_key_value_heads=max(1, z["heads"] // 4), head_dim=z["width"] // z["heads"],
+        rms_norm_eps=1e-5, rope_theta=10000.0, max_position_embeddings=8192, tie_word_embeddings=True))
+    return zcfg, lcfg
+
+
+def measure_designs(args) -> int:
+    """Decode (batch ``--batch``, contexts of ``--context``) and a 2,048-token prefill of Zifelorn beside Llama at
+    equal sizes, through LLMEngine.step, random weights; one JSON line."""
+    import torch
+    from mini_inference_engine_amd import LLMEngine
+    from mini_inference_engine_amd.config import EngineConfig
+    from mini_inference_engine_amd.weights import random_tensors
+    context = args.context or 1024
+    out = {"metric": "design_comparison", "dtype": "bf16", "data": "synthetic: random weights, uniform random token ids",
+           "batch": args.batch, "context": context, "steps": args.steps, "sizes": {}}
+    for size in (args.design_sizes.split(",") if args.design_sizes else DESIGN_SIZES):
+        row = {}
+        for name, cfg in zip(("zifelorn", "llama"), design_configs(size, args.layers or 1)):
+            weights = random_tensors(cfg, args.seed, torch.bfloat16, std=0.02, device="cuda")
+            pages = args.batch * (-(-max(context, 2048) // args.block_size)) + 1 + 64
+            ecfg = EngineConfig(block_size=args.block_size, max_num_seqs=args.batch, max_num_batched_tokens=2048,
+                                max_model_len=max(context, 2048), num_blocks=pages, use_hip_graphs=not args.no_graphs,
+                                graph_batch_sizes=(args.batch,))
+            eng = LLMEngine(cfg, ecfg, dtype=torch.bfloat16, verbose=False, weights=weights)
+            eng.model_cfg_vocab = getattr(cfg, "vocab_size", None) or cfg.vocab
+            dt, captured, ctx = measure_decode(eng, args.batch, context, args.steps, args.warmup, args.seed, vocab=eng.model_cfg_vocab)
+            t = measure_prefill(eng, 2048, args.seed + 100, vocab=eng.model_cfg_vocab)
+            row[name] = {"layers": 4 * (args.layers or 1), "decode_tok_s": round(args.batch * args.steps / dt, 1),
+                         "decode_ms_per_step": round(dt / args.steps * 1e3, 4), "captured_steps": captured,
+                         "prefill_2048_tok_s": round(2048 / t, 1), "prefill_ms": round(t * 1e3, 3),
+                         "weight_MB": round(eng.runner.model.weight_bytes() / 1e6, 1)}
+            del eng, weights
+            torch.cuda.empty_cache()
+        out["sizes"][size] = row
+    print(json.dumps(out), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
+    ap.add_argument("--design", choices=["zifelorn"], default=None,
+                    help="instead of the default workload: Zifelorn beside Llama at equal layer sizes (decode and prefill)")
+    ap.add_argument("--design-sizes", default=None, help="comma-separated widths of --design (default: all of 1024, 2048)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
@@ -445,6 +507,9 @@ def main() -> int:
         if int(os.environ.get("RANK", "0")) == 0:
             print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported", flush=True)
         return 2
+
+    if args.design:
+        return measure_designs(args)
 
     import torch
     from mini_inference_engine_amd import LLMEngine

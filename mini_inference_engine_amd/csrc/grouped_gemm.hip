@@ -117,6 +117,107 @@ grouped_gemm_kernel(GroupedArgs p) {
   }
 }
 
+// The same product for bfloat16 operands on the matrix cores (v_mfma_f32_16x16x32_bf16).  A workgroup of 4 waves
+// owns a 64 x 64 tile of C; a k-step of 32 brings 64 rows x 32 k of A and of W into the LDS in 16-byte pieces
+// (row r, k-block b at slot 4 r + (b ^ (r / 4) % 4), which spreads the fragment reads over the banks) while the
+// next k-step's pieces are already on their way into registers; wave w multiplies the four 16-row tiles of A
+// with its own 16 weight rows.  Every output is the same chain of matrix instructions in increasing k wherever
+// its tile lies, so a row's result does not depend on the rows beside it.  K, the row strides and the group
+// offsets are multiples of 8 and the operands 16-byte aligned (checked by the caller).
+typedef __bf16 gg_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float gg_f32x4 __attribute__((ext_vector_type(4)));
+union GGFrag {
+  gg_bf16x8 v;
+  uint4 q;
+};
+
+template <typename TC>
+__global__ void __launch_bounds__(256)
+grouped_gemm_mfma_kernel(GroupedArgs p) {
+  __shared__ uint4 As[256];
+  __shared__ uint4 Ws[256];
+  __shared__ int a_rows[GG_T];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * GG_T;
+  int g, m0, m_end, c_row0;
+  if (p.offs) {
+    int tile = blockIdx.y, start = 0, cnt = 0;
+    for (g = 0; g < p.G; ++g) {
+      start = p.offs[g];
+      cnt = p.offs[g + 1] - start;
+      const int nt = (cnt + GG_T - 1) / GG_T;
+      if (tile < nt) break;
+      tile -= nt;
+    }
+    if (g == p.G) return;
+    m0 = tile * GG_T;
+    m_end = cnt;
+    c_row0 = start;
+    if (tid < GG_T) {
+      const int r = m0 + tid;
+      a_rows[tid] = r < cnt ? (p.gather ? p.gather[start + r] / p.gather_div : start + r) : -1;
+    }
+  } else {
+    g = blockIdx.z;
+    m0 = blockIdx.y * GG_T;
+    m_end = p.M;
+    c_row0 = 0;
+    if (tid < GG_T) a_rows[tid] = m0 + tid < p.M ? m0 + tid : -1;
+  }
+  __syncthreads();
+  const bf16* A = (const bf16*)p.A + (size_t)(g % p.a_mod) * p.a_group;
+  const bf16* W = (const bf16*)p.W + (size_t)g * p.w_group;
+  // the piece this thread brings in: row tid / 4, k-block tid % 4
+  const int lrow = tid >> 2, lkb = tid & 3;
+  const int ar = a_rows[lrow];
+  const bf16* a_src = ar >= 0 ? A + (size_t)ar * p.lda + lkb * 8 : nullptr;
+  const bf16* w_src = n0 + lrow < p.N ? W + (size_t)(n0 + lrow) * p.ldw + lkb * 8 : nullptr;
+  const int put = lrow * 4 + (lkb ^ ((lrow >> 2) & 3));
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  auto fetch = [&](const bf16* src, int k0) { return src && k0 + lkb * 8 < p.K ? *reinterpret_cast<const uint4*>(src + k0) : zero; };
+  const int col = lane & 15, kb = lane >> 4;
+  const int wr = wave * 16 + col;
+  const int w_get = wr * 4 + (kb ^ ((wr >> 2) & 3));
+  gg_f32x4 acc[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) acc[mt] = gg_f32x4{0.f, 0.f, 0.f, 0.f};
+  uint4 ra = fetch(a_src, 0), rw = fetch(w_src, 0);
+  for (int k0 = 0; k0 < p.K; k0 += 32) {
+    As[put] = ra;
+    Ws[put] = rw;
+    __syncthreads();
+    if (k0 + 32 < p.K) {
+      ra = fetch(a_src, k0 + 32);
+      rw = fetch(w_src, k0 + 32);
+    }
+    GGFrag b;
+    b.q = Ws[w_get];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+      const int r = mt * 16 + col;
+      GGFrag a;
+      a.q = As[r * 4 + (kb ^ ((r >> 2) & 3))];
+      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[mt], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+  TC* C = (TC*)p.C + (size_t)g * p.c_group;
+  const int n = n0 + wave * 16 + col;
+  if (n >= p.N) return;
+  const float bias = p.bias ? p.bias[(size_t)g * p.N + n] : 0.f;
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = m0 + mt * 16 + kb * 4 + i;
+      if (m >= m_end) continue;
+      const size_t crow = (size_t)(c_row0 + m);
+      float v = mie_act(acc[mt][i] + bias, p.act);
+      if (p.gate) v *= mie_sigmoid(p.gate[crow * p.ldg + (size_t)g * p.N + n]);
+      C[crow * p.ldc + n] = from_float<TC>(v);
+    }
+}
+
 MIE_EXPORT const char* grouped_gemm_last_error() { return g_mie_error; }
 
 template <typename TA, typename TW>
@@ -149,6 +250,16 @@ MIE_EXPORT int mie_grouped_linear(const void* A, int a_dtype, long lda, long a_g
   const long mt = (M + GG_T - 1) / GG_T + (offs ? G : 0);
   if (mt > 65535 || G > 65535) MIE_FAIL("grouped_linear: %ld row tiles, %d groups are beyond the grid", mt, G);
   dim3 grid((N + GG_T - 1) / GG_T, (unsigned)mt, offs ? 1 : G);
+  // bfloat16 operands that the matrix-core kernel's 16-byte loads can take
+  if (a_dtype == MIE_BF16 && w_dtype == MIE_BF16 && (c_dtype == MIE_BF16 || c_dtype == MIE_F32) && K % 8 == 0 && lda % 8 == 0 &&
+      ldw % 8 == 0 && p.a_group % 8 == 0 && w_group % 8 == 0 && (((uintptr_t)A | (uintptr_t)W) & 15) == 0) {
+    if (c_dtype == MIE_BF16)
+      hipLaunchKernelGGL(grouped_gemm_mfma_kernel<bf16>, grid, dim3(256), 0, s, p);
+    else
+      hipLaunchKernelGGL(grouped_gemm_mfma_kernel<float>, grid, dim3(256), 0, s, p);
+    MIE_CHECK_LAUNCH("grouped_linear");
+    return 0;
+  }
   if (a_dtype == MIE_F32 && w_dtype == MIE_F32) return launch_grouped<float, float>(p, c_dtype, grid, s);
   if (a_dtype == MIE_F32 && w_dtype == MIE_BF16) return launch_grouped<float, bf16>(p, c_dtype, grid, s);
   if (a_dtype == MIE_BF16 && w_dtype == MIE_F32) return launch_grouped<bf16, float>(p, c_dtype, grid, s);
