@@ -26,6 +26,7 @@ struct GroupedArgs {
   const int* offs;              // rows shape: [G + 1]; null: columns shape
   const int* gather; int gather_div;
   int M, N, K, G, act;
+  const void* zeros;            // 64 bytes of zeros in device memory: what a load beyond a tile's rows or beyond K reads
 };
 
 template <typename TA, typename TW, typename TC>
@@ -131,91 +132,262 @@ union GGFrag {
   uint4 q;
 };
 
-template <typename TC>
+// TM x TN: the tile of C a workgroup owns; its four waves lie 2 x 2 over it, each with (TM / 32) x (TN / 32) tiles of
+// 16 x 16.  Two LDS buffers: while k-step i is multiplied, the pieces of k-step i + 1 are on their way into registers
+// and go into the other buffer before the one barrier of the step.
+template <int TM, int TN, typename TC>
 __global__ void __launch_bounds__(256)
 grouped_gemm_mfma_kernel(GroupedArgs p) {
-  __shared__ uint4 As[256];
-  __shared__ uint4 Ws[256];
-  __shared__ int a_rows[GG_T];
+  constexpr int MT = TM / 32, NT = TN / 32;          // 16-row / 16-column tiles a wave
+  constexpr int PA = TM * 4 / 256, PW = TN * 4 / 256;  // 16-byte pieces of A / W a thread brings in per k-step
+  __shared__ uint4 As[2][TM * 4];
+  __shared__ uint4 Ws[2][TN * 4];
+  __shared__ int a_rows[TM];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * GG_T;
+  const int n0 = blockIdx.x * TN;
   int g, m0, m_end, c_row0;
   if (p.offs) {
     int tile = blockIdx.y, start = 0, cnt = 0;
     for (g = 0; g < p.G; ++g) {
       start = p.offs[g];
       cnt = p.offs[g + 1] - start;
-      const int nt = (cnt + GG_T - 1) / GG_T;
+      const int nt = (cnt + TM - 1) / TM;
       if (tile < nt) break;
       tile -= nt;
     }
     if (g == p.G) return;
-    m0 = tile * GG_T;
+    m0 = tile * TM;
     m_end = cnt;
     c_row0 = start;
-    if (tid < GG_T) {
+    for (int i = tid; i < TM; i += 256) {
+      const int r = m0 + i;
+      a_rows[i] = r < cnt ? (p.gather ? p.gather[start + r] / p.gather_div : start + r) : -1;
+    }
+  } else {
+    g = blockIdx.z;
+    m0 = blockIdx.y * TM;
+    m_end = p.M;
+    c_row0 = 0;
+    for (int i = tid; i < TM; i += 256) a_rows[i] = m0 + i < p.M ? m0 + i : -1;
+  }
+  __syncthreads();
+  const bf16* A = (const bf16*)p.A + (size_t)(g % p.a_mod) * p.a_group;
+  const bf16* W = (const bf16*)p.W + (size_t)g * p.w_group;
+  // piece j of this thread: row (tid + 256 j) / 4, k-block tid % 4
+  const int lkb = tid & 3;
+  const bf16* a_src[PA];
+  const bf16* w_src[PW];
+  int a_put[PA], w_put[PW];
+#pragma unroll
+  for (int j = 0; j < PA; ++j) {
+    const int row = (tid >> 2) + 64 * j, ar = a_rows[row];
+    a_src[j] = ar >= 0 ? A + (size_t)ar * p.lda + lkb * 8 : nullptr;
+    a_put[j] = row * 4 + (lkb ^ ((row >> 2) & 3));
+  }
+#pragma unroll
+  for (int j = 0; j < PW; ++j) {
+    const int row = (tid >> 2) + 64 * j;
+    w_src[j] = n0 + row < p.N ? W + (size_t)(n0 + row) * p.ldw + lkb * 8 : nullptr;
+    w_put[j] = row * 4 + (lkb ^ ((row >> 2) & 3));
+  }
+  const uint4 zero = make_uint4(0, 0, 0, 0);
+  auto fetch = [&](const bf16* src, int k0) { return src && k0 + lkb * 8 < p.K ? *reinterpret_cast<const uint4*>(src + k0) : zero; };
+  const int col = lane & 15, kb = lane >> 4;
+  const int wm = (wave >> 1) * (TM / 2), wn = (wave & 1) * (TN / 2);
+  gg_f32x4 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j) acc[i][j] = gg_f32x4{0.f, 0.f, 0.f, 0.f};
+  uint4 ra[PA], rw[PW];
+#pragma unroll
+  for (int j = 0; j < PA; ++j) As[0][a_put[j]] = fetch(a_src[j], 0);
+#pragma unroll
+  for (int j = 0; j < PW; ++j) Ws[0][w_put[j]] = fetch(w_src[j], 0);
+  __syncthreads();
+  int cur = 0;
+  for (int k0 = 0; k0 < p.K; k0 += 32) {
+    const bool more = k0 + 32 < p.K;
+    if (more) {
+#pragma unroll
+      for (int j = 0; j < PA; ++j) ra[j] = fetch(a_src[j], k0 + 32);
+#pragma unroll
+      for (int j = 0; j < PW; ++j) rw[j] = fetch(w_src[j], k0 + 32);
+    }
+    GGFrag a[MT], b[NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+      const int r = wm + i * 16 + col;
+      a[i].q = As[cur][r * 4 + (kb ^ ((r >> 2) & 3))];
+    }
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+      const int r = wn + j * 16 + col;
+      b[j].q = Ws[cur][r * 4 + (kb ^ ((r >> 2) & 3))];
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int j = 0; j < NT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[j].v, acc[i][j], 0, 0, 0);
+    if (more) {
+#pragma unroll
+      for (int j = 0; j < PA; ++j) As[cur ^ 1][a_put[j]] = ra[j];
+#pragma unroll
+      for (int j = 0; j < PW; ++j) Ws[cur ^ 1][w_put[j]] = rw[j];
+    }
+    __syncthreads();
+    cur ^= 1;
+  }
+  TC* C = (TC*)p.C + (size_t)g * p.c_group;
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int n = n0 + wn + j * 16 + col;
+    if (n >= p.N) continue;
+    const float bias = p.bias ? p.bias[(size_t)g * p.N + n] : 0.f;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int m = m0 + wm + i * 16 + kb * 4 + e;
+        if (m >= m_end) continue;
+        const size_t crow = (size_t)(c_row0 + m);
+        float v = mie_act(acc[i][j][e] + bias, p.act);
+        if (p.gate) v *= mie_sigmoid(p.gate[crow * p.ldg + (size_t)g * p.N + n]);
+        C[crow * p.ldc + n] = from_float<TC>(v);
+      }
+  }
+}
+
+// Tiles of 128 x 128 for steps of many rows: the k-steps come into a ring of three LDS stages by loads that write the
+// LDS directly (no registers in between, two stages on their way while the third is multiplied), 1 KB a fragment of
+// 16 rows x 32 k: lane l brings k-block (l % 4) ^ (l / 16) % 4 of row l / 4, which is the slot order above.  A lane
+// whose row or k-block does not exist reads from a block of zeros instead, so every wave issues the same four loads a
+// stage and one count tells when a stage has landed.  The fragments are read back in one piece of assembly with its
+// own wait: the compiler does not know of the loads that write the LDS.
+#define GG_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+typedef uint32_t gg_u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void gg_read4(uint32_t base, gg_u32x4 (&f)[4]) {
+  asm volatile(
+    "ds_read_b128 %0, %4\n\t"
+    "ds_read_b128 %1, %4 offset:1024\n\t"
+    "ds_read_b128 %2, %4 offset:2048\n\t"
+    "ds_read_b128 %3, %4 offset:3072\n\t"
+    "s_waitcnt lgkmcnt(0)"
+    : "=&v"(f[0]), "=&v"(f[1]), "=&v"(f[2]), "=&v"(f[3])
+    : "v"(base)
+    : "memory");
+}
+
+template <typename TC>
+__global__ void __launch_bounds__(256)
+grouped_gemm_ring_kernel(GroupedArgs p) {
+  constexpr int TM = 128, TN = 128, STAGES = 3, STAGE_BYTES = (TM + TN) * 64;
+  __shared__ __align__(16) char lds[STAGES * STAGE_BYTES];
+  __shared__ int a_rows[TM];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int n0 = blockIdx.x * TN;
+  int g, m0, m_end, c_row0;
+  if (p.offs) {
+    int tile = blockIdx.y, start = 0, cnt = 0;
+    for (g = 0; g < p.G; ++g) {
+      start = p.offs[g];
+      cnt = p.offs[g + 1] - start;
+      const int nt = (cnt + TM - 1) / TM;
+      if (tile < nt) break;
+      tile -= nt;
+    }
+    if (g == p.G) return;
+    m0 = tile * TM;
+    m_end = cnt;
+    c_row0 = start;
+    if (tid < TM) {
       const int r = m0 + tid;
       a_rows[tid] = r < cnt ? (p.gather ? p.gather[start + r] / p.gather_div : start + r) : -1;
     }
   } else {
     g = blockIdx.z;
-    m0 = blockIdx.y * GG_T;
+    m0 = blockIdx.y * TM;
     m_end = p.M;
     c_row0 = 0;
-    if (tid < GG_T) a_rows[tid] = m0 + tid < p.M ? m0 + tid : -1;
+    if (tid < TM) a_rows[tid] = m0 + tid < p.M ? m0 + tid : -1;
   }
   __syncthreads();
   const bf16* A = (const bf16*)p.A + (size_t)(g % p.a_mod) * p.a_group;
   const bf16* W = (const bf16*)p.W + (size_t)g * p.w_group;
-  // the piece this thread brings in: row tid / 4, k-block tid % 4
-  const int lrow = tid >> 2, lkb = tid & 3;
-  const int ar = a_rows[lrow];
-  const bf16* a_src = ar >= 0 ? A + (size_t)ar * p.lda + lkb * 8 : nullptr;
-  const bf16* w_src = n0 + lrow < p.N ? W + (size_t)(n0 + lrow) * p.ldw + lkb * 8 : nullptr;
-  const int put = lrow * 4 + (lkb ^ ((lrow >> 2) & 3));
-  const uint4 zero = make_uint4(0, 0, 0, 0);
-  auto fetch = [&](const bf16* src, int k0) { return src && k0 + lkb * 8 < p.K ? *reinterpret_cast<const uint4*>(src + k0) : zero; };
-  const int col = lane & 15, kb = lane >> 4;
-  const int wr = wave * 16 + col;
-  const int w_get = wr * 4 + (kb ^ ((wr >> 2) & 3));
-  gg_f32x4 acc[4];
+  // what this lane brings in: fragments 2 wave and 2 wave + 1 of A and of W, row lane / 4 of each
+  const int lrow = lane >> 2, lkb = (lane & 3) ^ ((lane >> 4) & 3);
+  const bf16* zero_lane = (const bf16*)p.zeros + lkb * 8;
+  const bf16* src[4];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) acc[mt] = gg_f32x4{0.f, 0.f, 0.f, 0.f};
-  uint4 ra = fetch(a_src, 0), rw = fetch(w_src, 0);
-  for (int k0 = 0; k0 < p.K; k0 += 32) {
-    As[put] = ra;
-    Ws[put] = rw;
-    __syncthreads();
-    if (k0 + 32 < p.K) {
-      ra = fetch(a_src, k0 + 32);
-      rw = fetch(w_src, k0 + 32);
-    }
-    GGFrag b;
-    b.q = Ws[w_get];
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-      const int r = mt * 16 + col;
-      GGFrag a;
-      a.q = As[r * 4 + (kb ^ ((r >> 2) & 3))];
-      acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[mt], 0, 0, 0);
-    }
-    __syncthreads();
+  for (int j = 0; j < 2; ++j) {
+    const int ar = a_rows[(2 * wave + j) * 16 + lrow];
+    src[j] = ar >= 0 ? A + (size_t)ar * p.lda + lkb * 8 : nullptr;
+    const int n = n0 + (2 * wave + j) * 16 + lrow;
+    src[2 + j] = n < p.N ? W + (size_t)n * p.ldw + lkb * 8 : nullptr;
   }
-  TC* C = (TC*)p.C + (size_t)g * p.c_group;
-  const int n = n0 + wave * 16 + col;
-  if (n >= p.N) return;
-  const float bias = p.bias ? p.bias[(size_t)g * p.N + n] : 0.f;
+  auto issue = [&](int s) {
+    char* base = lds + (s % STAGES) * STAGE_BYTES;
+    const int k0 = s * 32;
+    const bool kok = k0 + lkb * 8 < p.K;
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int m = m0 + mt * 16 + kb * 4 + i;
-      if (m >= m_end) continue;
-      const size_t crow = (size_t)(c_row0 + m);
-      float v = mie_act(acc[mt][i] + bias, p.act);
-      if (p.gate) v *= mie_sigmoid(p.gate[crow * p.ldg + (size_t)g * p.N + n]);
-      C[crow * p.ldc + n] = from_float<TC>(v);
+    for (int j = 0; j < 4; ++j) {
+      const bf16* from = src[j] && kok ? src[j] + k0 : zero_lane;
+      const int frag = (j < 2 ? 0 : TM / 16) + 2 * wave + (j & 1);
+      __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)from,
+                                       (__attribute__((address_space(3))) void*)(base + frag * 1024), 16, 0, 0);
     }
+  };
+  const int col = lane & 15, kb = lane >> 4;
+  const int rslot = col * 4 + (kb ^ ((col >> 2) & 3));
+  const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
+  const uint32_t a_off = (wave >> 1) * 4096 + rslot * 16, b_off = TM * 64 + (wave & 1) * 4096 + rslot * 16;
+  gg_f32x4 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = gg_f32x4{0.f, 0.f, 0.f, 0.f};
+  const int nk = (p.K + 31) / 32;
+  issue(0);
+  issue(1);
+  for (int it = 0; it < nk; ++it) {
+    GG_VMCNT(4);                       // this wave's loads of stage `it` have landed
+    __builtin_amdgcn_s_barrier();      // and everybody else's; everybody is done reading stage it - 1
+    issue(it + 2);                     // into the buffer stage it - 1 used (zeros beyond K)
+    const uint32_t base = lds0 + (it % STAGES) * STAGE_BYTES;
+    gg_u32x4 fa[4], fb[4];
+    gg_read4(base + a_off, fa);
+    gg_read4(base + b_off, fb);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        GGFrag a, b;
+        a.q = *reinterpret_cast<uint4*>(&fa[i]);
+        b.q = *reinterpret_cast<uint4*>(&fb[j]);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, acc[i][j], 0, 0, 0);
+      }
+  }
+  GG_VMCNT(0);                         // nothing of this wave may still be writing the LDS when it ends
+  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  TC* C = (TC*)p.C + (size_t)g * p.c_group;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + wn + j * 16 + col;
+    if (n >= p.N) continue;
+    const float bias = p.bias ? p.bias[(size_t)g * p.N + n] : 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int m = m0 + wm + i * 16 + kb * 4 + e;
+        if (m >= m_end) continue;
+        const size_t crow = (size_t)(c_row0 + m);
+        float v = mie_act(acc[i][j][e] + bias, p.act);
+        if (p.gate) v *= mie_sigmoid(p.gate[crow * p.ldg + (size_t)g * p.N + n]);
+        C[crow * p.ldc + n] = from_float<TC>(v);
+      }
+  }
 }
 
 MIE_EXPORT const char* grouped_gemm_last_error() { return g_mie_error; }
@@ -232,12 +404,13 @@ static int launch_grouped(const GroupedArgs& p, int c_dtype, dim3 grid, hipStrea
   return 0;
 }
 
-// Strides and group offsets are in elements.  Rows shape: offs non-null, M = the length of the sorted list (an upper
+// Strides and group offsets are in elements.  zeros: 64 bytes of zeros in device memory (or null: the kernels that
+// need them are not used).  Rows shape: offs non-null, M = the length of the sorted list (an upper
 // bound of any group's rows), a_group / c_group / a_mod unused.
 MIE_EXPORT int mie_grouped_linear(const void* A, int a_dtype, long lda, long a_group, int a_mod, const void* W, int w_dtype,
                                   long ldw, long w_group, void* C, int c_dtype, long ldc, long c_group, const float* bias,
                                   const float* gate, long ldg, const int* offs, const int* gather, int gather_div, int M,
-                                  int N, int K, int G, int act, hipStream_t s) {
+                                  int N, int K, int G, int act, const void* zeros, hipStream_t s) {
   if (M <= 0 || N <= 0 || G <= 0) return 0;
   if (K <= 0 || !A || !W || !C) MIE_FAIL("grouped_linear: K %d or a null operand", K);
   if (lda < K && !offs && a_group == 0) MIE_FAIL("grouped_linear: A row stride %ld < K %d", lda, K);
@@ -246,17 +419,25 @@ MIE_EXPORT int mie_grouped_linear(const void* A, int a_dtype, long lda, long a_g
   if (gather && gather_div <= 0) MIE_FAIL("grouped_linear: gather divisor %d", gather_div);
   if (act < MIE_ACT_NONE || act > MIE_ACT_RELU2) MIE_FAIL("grouped_linear: activation code %d", act);
   GroupedArgs p = {A, lda, offs ? 0 : a_group, offs ? 1 : a_mod, W, ldw, w_group, C, ldc, offs ? 0 : c_group, bias, gate, ldg,
-                   offs, gather, gather_div, M, N, K, G, act};
+                   offs, gather, gather_div, M, N, K, G, act, zeros};
   const long mt = (M + GG_T - 1) / GG_T + (offs ? G : 0);
   if (mt > 65535 || G > 65535) MIE_FAIL("grouped_linear: %ld row tiles, %d groups are beyond the grid", mt, G);
   dim3 grid((N + GG_T - 1) / GG_T, (unsigned)mt, offs ? 1 : G);
-  // bfloat16 operands that the matrix-core kernel's 16-byte loads can take
+  // bfloat16 operands that the matrix-core kernel's 16-byte loads can take: tiles of 128 x 128 where there are rows
+  // enough to fill them (a function of the step's size, not of a row's place in it), of 64 x 64 otherwise
   if (a_dtype == MIE_BF16 && w_dtype == MIE_BF16 && (c_dtype == MIE_BF16 || c_dtype == MIE_F32) && K % 8 == 0 && lda % 8 == 0 &&
       ldw % 8 == 0 && p.a_group % 8 == 0 && w_group % 8 == 0 && (((uintptr_t)A | (uintptr_t)W) & 15) == 0) {
-    if (c_dtype == MIE_BF16)
-      hipLaunchKernelGGL(grouped_gemm_mfma_kernel<bf16>, grid, dim3(256), 0, s, p);
-    else
-      hipLaunchKernelGGL(grouped_gemm_mfma_kernel<float>, grid, dim3(256), 0, s, p);
+    const bool big = zeros && (offs ? M >= 128L * G : M >= 256);
+    const int T = big ? 128 : 64;
+    const long mtiles = (M + T - 1) / T + (offs ? G : 0);
+    if (mtiles > 65535) MIE_FAIL("grouped_linear: %ld row tiles are beyond the grid", mtiles);
+    dim3 mgrid((N + T - 1) / T, (unsigned)mtiles, offs ? 1 : G);
+#define GG_MFMA(T_, TC_) hipLaunchKernelGGL((grouped_gemm_mfma_kernel<T_, T_, TC_>), mgrid, dim3(256), 0, s, p)
+    if (big && c_dtype == MIE_BF16) hipLaunchKernelGGL(grouped_gemm_ring_kernel<bf16>, mgrid, dim3(256), 0, s, p);
+    else if (big) hipLaunchKernelGGL(grouped_gemm_ring_kernel<float>, mgrid, dim3(256), 0, s, p);
+    else if (c_dtype == MIE_BF16) GG_MFMA(64, bf16);
+    else GG_MFMA(64, float);
+#undef GG_MFMA
     MIE_CHECK_LAUNCH("grouped_linear");
     return 0;
   }

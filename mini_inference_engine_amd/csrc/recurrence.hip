@@ -63,7 +63,103 @@ rglru_scan_kernel(const float* __restrict__ u, const float* __restrict__ gates, 
   }
 }
 
+// Rows of many tokens: the same recurrence in chunks of L tokens that run side by side.  S_t = a_t S_{t-1} + b_t is
+// linear in S, so a chunk is summed up by (A, B) with S_end = A S_start + B.  Pass 1: every (row, chunk, channel)
+// computes its A and B (and chunk 0 notes the state the row starts from); pass 2: every chunk folds the
+// summaries of the chunks before it, in order, onto the start state and runs its tokens from there; the last
+// chunk of a row leaves the state and the convolution's tail.  Each value comes out of the same chain of
+// operations as in the one-pass kernel except for the fold over whole chunks.
+struct ScanArgs {
+  const float* u; const float* gates; const float* lam; const float* y; long ldy; const float* y_bias; const float* x; long ldx;
+  const float* x_bias; float* state; float* tail; const int* row_start; const int* slots; void* out; float* chunk_a;
+  float* chunk_b; float* start; int C, K, L, max_chunks; float decay_scale;
+};
+
+__device__ __forceinline__ void rglru_step(const ScanArgs& p, int t, int c, float sp, float& a, float& b) {
+  const float rg = mie_sigmoid(p.gates[(size_t)t * 2 * p.C + c]);
+  const float ig = mie_sigmoid(p.gates[(size_t)t * 2 * p.C + p.C + c]);
+  const float log_a = -sp * rg;
+  a = expf(log_a);
+  b = sqrtf(-expm1f(2.0f * log_a)) * ig * p.u[(size_t)t * p.C + c];
+}
+
+template <int PASS, typename TO>
+__global__ void __launch_bounds__(256)
+rglru_chunk_kernel(ScanArgs p) {
+  const int r = blockIdx.x / p.max_chunks, j = blockIdx.x - r * p.max_chunks, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= p.C) return;
+  const int a0 = p.row_start[r], b0 = p.row_start[r + 1], slot = p.slots[r];
+  const int t0 = a0 + j * p.L;
+  if (t0 >= b0) return;
+  const int t1 = t0 + p.L < b0 ? t0 + p.L : b0;
+  const float lm = p.lam[c];
+  const float sp = p.decay_scale * (lm > 20.f ? lm : log1pf(expf(lm)));
+  const size_t at = ((size_t)r * p.max_chunks + j) * p.C + c;
+  if (PASS == 1) {
+    float A = 1.f, B = 0.f;
+    for (int t = t0; t < t1; ++t) {
+      float a, b;
+      rglru_step(p, t, c, sp, a, b);
+      B = fmaf(a, B, b);
+      A *= a;
+    }
+    p.chunk_a[at] = A;
+    p.chunk_b[at] = B;
+    if (j == 0) p.start[(size_t)r * p.C + c] = p.state[(size_t)slot * p.C + c];
+    return;
+  }
+  float S = p.start[(size_t)r * p.C + c];
+  for (int i = 0; i < j; ++i) {
+    const size_t e = ((size_t)r * p.max_chunks + i) * p.C + c;
+    S = fmaf(p.chunk_a[e], S, p.chunk_b[e]);
+  }
+  const float yb = p.y_bias[c];
+  TO* out = (TO*)p.out;
+  for (int t = t0; t < t1; ++t) {
+    float a, b;
+    rglru_step(p, t, c, sp, a, b);
+    S = fmaf(a, S, b);
+    out[(size_t)t * p.C + c] = from_float<TO>(S * mie_gelu_tanh(p.y[(size_t)t * p.ldy + c] + yb));
+  }
+  if (t1 != b0) return;
+  p.state[(size_t)slot * p.C + c] = S;
+  const int n = b0 - a0, keep = p.K - 1;
+  float* tl = p.tail + (size_t)slot * (keep > 0 ? keep : 1) * p.C;
+  const float xb = p.x_bias[c];
+  for (int i = 0; i < keep; ++i) {
+    const int src = n + i;
+    tl[(size_t)i * p.C + c] = src < keep ? tl[(size_t)src * p.C + c] : p.x[(size_t)(a0 + src - keep) * p.ldx + c] + xb;
+  }
+}
+
 MIE_EXPORT const char* recurrence_last_error() { return g_mie_error; }
+
+// The chunked form for steps whose longest row has max_row_tokens tokens: chunk_a, chunk_b [rows, max_chunks, C] and
+// start [rows, C] are scratch, max_chunks = ceil(max_row_tokens / chunk).
+MIE_EXPORT int mie_rglru_scan_chunked(const float* u, const float* gates, const float* lam, const float* y, long ldy,
+                                      const float* y_bias, const float* x, long ldx, const float* x_bias, float* state,
+                                      float* tail, const int* row_start, const int* slots, void* out, int out_dtype, int rows,
+                                      int C, int K, float decay_scale, int chunk, int max_chunks, float* chunk_a, float* chunk_b,
+                                      float* start, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (C <= 0 || K <= 0 || ldy < C || ldx < C || chunk <= 0 || max_chunks <= 0)
+    MIE_FAIL("rglru_scan_chunked: %d channels, %d taps, row strides %ld, %ld, chunks of %d x %d", C, K, ldy, ldx, chunk, max_chunks);
+  if (!u || !gates || !lam || !y || !y_bias || !x || !x_bias || !state || !tail || !row_start || !slots || !out || !chunk_a ||
+      !chunk_b || !start)
+    MIE_FAIL("rglru_scan_chunked: operands");
+  if ((long)rows * max_chunks > 2000000000L) MIE_FAIL("rglru_scan_chunked: %d rows of %d chunks are beyond the grid", rows, max_chunks);
+  if (out_dtype != MIE_F32 && out_dtype != MIE_BF16) MIE_FAIL("rglru_scan_chunked: output dtype code %d", out_dtype);
+  ScanArgs p = {u, gates, lam, y, ldy, y_bias, x, ldx, x_bias, state, tail, row_start, slots, out, chunk_a, chunk_b, start,
+                C, K, chunk, max_chunks, decay_scale};
+  dim3 grid(rows * max_chunks, (C + 255) / 256);
+  hipLaunchKernelGGL((rglru_chunk_kernel<1, float>), grid, dim3(256), 0, s, p);
+  if (out_dtype == MIE_F32)
+    hipLaunchKernelGGL((rglru_chunk_kernel<2, float>), grid, dim3(256), 0, s, p);
+  else
+    hipLaunchKernelGGL((rglru_chunk_kernel<2, bf16>), grid, dim3(256), 0, s, p);
+  MIE_CHECK_LAUNCH("rglru_scan_chunked");
+  return 0;
+}
 
 // x points at the first of the C input columns (rows ldx floats apart); taps [C, K]; tail [slots, max(1, K - 1), C].
 MIE_EXPORT int mie_causal_conv(const float* x, long ldx, const float* in_bias, const float* taps, const float* conv_bias,

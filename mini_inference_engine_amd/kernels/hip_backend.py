@@ -458,10 +458,12 @@ class HipBackend(KernelBackend):
     def _grouped(self, A, lda, a_group, a_mod, W, ldw, w_group, C, ldc, c_group, M, N, K, G, bias=None, gate=None, ldg=0,
                  offs=None, gather=None, gather_div=1, act="none"):
         lib = self.lib("grouped_gemm")
+        if self._zeros is None:
+            self._zeros = torch.zeros(64, dtype=torch.int32, device=W.device)
         library.check(lib, lib.mie_grouped_linear(
             _ptr(A), _code(A.dtype), lda, a_group, a_mod, _ptr(W), _code(W.dtype), ldw, w_group, _ptr(C), _code(C.dtype), ldc,
             c_group, _ptr(bias), gate, ldg, _ptr(offs), _ptr(gather), gather_div, M, N, K, G, self.ACT_CODES[act],
-            self._stream()))
+            _ptr(self._zeros), self._stream()))
 
     def grouped_linear(self, x, w, bias=None, x_groups=None):
         self._on_device(x, w, bias)
@@ -539,6 +541,8 @@ class HipBackend(KernelBackend):
         return out
 
     # ---- gated linear recurrence
+    SCAN_CHUNK = 32          # tokens a chunk of the recurrence's scan; rows up to this long run in one pass
+
     def _check_rows(self, what, step, T):
         for name, t, n in (("token_row", step.token_row, T), ("row_start", step.row_start, step.num_rows + 1),
                            ("state_slots", step.state_slots, step.num_rows)):
@@ -591,6 +595,19 @@ class HipBackend(KernelBackend):
             raise ValueError("rglru_scan: a state slot beyond the state's slots")
         out = torch.empty((T, C), dtype=self.act_dtype, device=u.device)
         lib = self.lib("recurrence")
+        longest = int(getattr(step, "max_row_tokens", 0) or (step.host["row_start"][1:] - step.host["row_start"][:-1]).max())
+        if longest > self.SCAN_CHUNK:
+            # rows of many tokens: chunks side by side (whether a step takes this path depends on its longest row
+            # alone; the two paths differ by the rounding of the fold over whole chunks)
+            chunks = -(-longest // self.SCAN_CHUNK)
+            scratch = torch.empty((2 * step.num_rows * chunks + step.num_rows, C), dtype=torch.float32, device=u.device)
+            n = step.num_rows * chunks
+            library.check(lib, lib.mie_rglru_scan_chunked(
+                _ptr(u), _ptr(gates), _ptr(lam), yp, y.stride(0), _ptr(y_bias), xp, x.stride(0), _ptr(x_bias), _ptr(state),
+                _ptr(tail), _ptr(step.row_start), _ptr(step.state_slots), _ptr(out), _code(out.dtype), step.num_rows, C, K,
+                float(decay_scale), self.SCAN_CHUNK, chunks, _ptr(scratch[:n]), _ptr(scratch[n:2 * n]), _ptr(scratch[2 * n:]),
+                self._stream()))
+            return out
         library.check(lib, lib.mie_rglru_scan(_ptr(u), _ptr(gates), _ptr(lam), yp, y.stride(0), _ptr(y_bias), xp, x.stride(0),
                                               _ptr(x_bias), _ptr(state), _ptr(tail), _ptr(step.row_start), _ptr(step.state_slots),
                                               _ptr(out), _code(out.dtype), step.num_rows, C, K, float(decay_scale), self._stream()))

@@ -26,7 +26,7 @@ register_kernel_module("gemm", {
     "mie_act_mul": [P, L, P, L, I, I, I, I, P],
 })
 register_kernel_module("grouped_gemm", {
-    "mie_grouped_linear": [P, I, L, L, I, P, I, L, L, P, I, L, L, P, P, L, P, P, I, I, I, I, I, I, P],
+    "mie_grouped_linear": [P, I, L, L, I, P, I, L, L, P, I, L, L, P, P, L, P, P, I, I, I, I, I, I, P, P],
     "mie_route_topk": [P, L, P, P, P, I, I, I, P],
     "mie_moe_align": [P, I, I, P, P, P, P],
     "mie_moe_combine": [P, P, P, P, I, I, I, P],
@@ -38,6 +38,7 @@ register_kernel_module("latent_attention", {
 register_kernel_module("recurrence", {
     "mie_causal_conv": [P, L, P, P, P, P, P, P, P, P, I, I, I, P],
     "mie_rglru_scan": [P, P, P, P, L, P, P, L, P, P, P, P, P, P, I, I, I, I, F, P],
+    "mie_rglru_scan_chunked": [P, P, P, P, L, P, P, L, P, P, P, P, P, P, I, I, I, I, F, I, I, P, P, P, P],
 })
 register_kernel_module("attention", {
     "mie_paged_attention": [P, L, P, P, P, I, P, I, P, P, I, I, I, I, I, F, I, P],

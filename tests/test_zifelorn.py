@@ -434,13 +434,13 @@ def test_gated_activation_kernel(hip, dtype, act):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_latent_attention_kernels(hip, dtype):
     ops, g = hip[dtype], torch.Generator().manual_seed(2)
-    for (H, dim, rot, vdim, r, n_freq, T) in ((3, 16, 8, 24, 40, 4, 37), (5, 8, 16, 8, 24, 4, 3), (2, 24, 4, 12, 28, 2, 130)):
+    for (H, dim, rot, vdim, r, n_freq, T) in ((3, 16, 8, 24, 40, 4, 37), (5, 8, 16, 8, 24, 4, 3), (2, 24, 4, 12, 28, 2, 130), (4, 32, 16, 40, 48, 8, 300)):
         P = -(-(r + rot) // 16) * 16
         inv_freq = (50.0 ** -(torch.arange(n_freq).double() * 2 / (2 * n_freq))).float().cuda()
         positions = torch.randint(0, 5000, (T,), generator=g).to(torch.int32).cuda()
         sums = _rand((T, 11 + r + rot + 5), torch.float32, g, 2.0)
         nw = _rand((r,), dtype, g) + 1
-        pages, page = 12, 16
+        pages, page = T // 16 + 3, 16
         slots = torch.randperm((pages - 1) * page, generator=g)[:T].to(torch.int32).cuda() + page
         kc = torch.full((pages, 1, page, P), 7.0, dtype=dtype).cuda()
         vc = torch.full((pages, 1, P, page), 7.0, dtype=dtype).cuda()
