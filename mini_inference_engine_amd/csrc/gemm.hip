@@ -93,8 +93,9 @@ __global__ void act_mul_kernel(const T* __restrict__ gu, long ld_in, T* __restri
 }
 
 // bfloat16 rows whose gate and up halves start on 16 bytes: eight values a thread and a load
+template <int ACT>
 __global__ void __launch_bounds__(256)
-silu_mul_bf16x8_kernel(const bf16* __restrict__ gu, long ld_in, bf16* __restrict__ out, long ld_out, int rows, int inter) {
+act_mul_bf16x8_kernel(const bf16* __restrict__ gu, long ld_in, bf16* __restrict__ out, long ld_out, int rows, int inter) {
   const int per_row = inter >> 3;
   const size_t total = (size_t)rows * per_row;
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
@@ -109,9 +110,20 @@ silu_mul_bf16x8_kernel(const bf16* __restrict__ gu, long ld_in, bf16* __restrict
       const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xFFFF0000u);
       // g / (1 + e^-g) by the hardware's exp2 and reciprocal (each within an ulp or two of the exact value, far
       // below the bfloat16 rounding that follows): a tenth of the instructions of expf and a division
-      const float s0 = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g0 * -1.4426950408889634f));
-      const float s1 = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g1 * -1.4426950408889634f));
-      const bf16 o0 = __float2bfloat16(g0 * s0 * u0), o1 = __float2bfloat16(g1 * s1 * u1);
+      float a0, a1;
+      if (ACT == MIE_ACT_SILU) {
+        a0 = g0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g0 * -1.4426950408889634f));
+        a1 = g1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g1 * -1.4426950408889634f));
+      } else if (ACT == MIE_ACT_GELU_TANH) {
+        // 0.5 z (1 + tanh(t)) = z / (1 + e^(-2 t)), t = sqrt(2 / pi) (z + 0.044715 z^3), by the same two instructions
+        const float t0 = 0.7978845608028654f * (g0 + 0.044715f * g0 * g0 * g0), t1 = 0.7978845608028654f * (g1 + 0.044715f * g1 * g1 * g1);
+        a0 = g0 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t0 * -2.8853900817779268f));
+        a1 = g1 * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(t1 * -2.8853900817779268f));
+      } else {
+        a0 = mie_act(g0, ACT);
+        a1 = mie_act(g1, ACT);
+      }
+      const bf16 o0 = __float2bfloat16(a0 * u0), o1 = __float2bfloat16(a1 * u1);
       ow[j] = (uint32_t)__builtin_bit_cast(uint16_t, o0) | ((uint32_t)__builtin_bit_cast(uint16_t, o1) << 16);
     }
     *reinterpret_cast<uint4*>(out + r * ld_out + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
@@ -161,7 +173,7 @@ MIE_EXPORT int mie_silu_mul(const void* gu, long ld_in, void* out, long ld_out, 
   else if (dtype == MIE_BF16 && (inter & 7) == 0 && (ld_in & 7) == 0 && (ld_out & 7) == 0 &&
            (((uintptr_t)gu | (uintptr_t)out) & 15) == 0) {
     int b8 = (int)((total / 8 + 255) / 256);
-    hipLaunchKernelGGL(silu_mul_bf16x8_kernel, dim3(b8 > 16384 ? 16384 : b8), dim3(256), 0, s, (const bf16*)gu, ld_in,
+    hipLaunchKernelGGL(act_mul_bf16x8_kernel<MIE_ACT_SILU>, dim3(b8 > 16384 ? 16384 : b8), dim3(256), 0, s, (const bf16*)gu, ld_in,
                        (bf16*)out, ld_out, rows, inter);
   } else if (dtype == MIE_BF16)
     hipLaunchKernelGGL(silu_mul_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (const bf16*)gu, ld_in, (bf16*)out, ld_out, rows, inter);
@@ -183,7 +195,15 @@ MIE_EXPORT int mie_act_mul(const void* gu, long ld_in, void* out, long ld_out, i
   if (blocks > 16384) blocks = 16384;
   if (dtype == MIE_F32)
     hipLaunchKernelGGL(act_mul_kernel<float>, dim3(blocks), dim3(256), 0, s, (const float*)gu, ld_in, (float*)out, ld_out, rows, inter, act);
-  else if (dtype == MIE_BF16)
+  else if (dtype == MIE_BF16 && (act == MIE_ACT_GELU_TANH || act == MIE_ACT_RELU2) && (inter & 7) == 0 && (ld_in & 7) == 0 &&
+           (ld_out & 7) == 0 && (((uintptr_t)gu | (uintptr_t)out) & 15) == 0) {
+    int b8 = (int)((total / 8 + 255) / 256);
+    b8 = b8 > 16384 ? 16384 : b8;
+    if (act == MIE_ACT_GELU_TANH)
+      hipLaunchKernelGGL(act_mul_bf16x8_kernel<MIE_ACT_GELU_TANH>, dim3(b8), dim3(256), 0, s, (const bf16*)gu, ld_in, (bf16*)out, ld_out, rows, inter);
+    else
+      hipLaunchKernelGGL(act_mul_bf16x8_kernel<MIE_ACT_RELU2>, dim3(b8), dim3(256), 0, s, (const bf16*)gu, ld_in, (bf16*)out, ld_out, rows, inter);
+  } else if (dtype == MIE_BF16)
     hipLaunchKernelGGL(act_mul_kernel<bf16>, dim3(blocks), dim3(256), 0, s, (const bf16*)gu, ld_in, (bf16*)out, ld_out, rows, inter, act);
   else
     MIE_FAIL("act_mul: dtype code %d", dtype);

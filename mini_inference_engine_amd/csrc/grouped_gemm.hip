@@ -118,13 +118,7 @@ grouped_gemm_kernel(GroupedArgs p) {
   }
 }
 
-// The same product for bfloat16 operands on the matrix cores (v_mfma_f32_16x16x32_bf16).  A workgroup of 4 waves
-// owns a 64 x 64 tile of C; a k-step of 32 brings 64 rows x 32 k of A and of W into the LDS in 16-byte pieces
-// (row r, k-block b at slot 4 r + (b ^ (r / 4) % 4), which spreads the fragment reads over the banks) while the
-// next k-step's pieces are already on their way into registers; wave w multiplies the four 16-row tiles of A
-// with its own 16 weight rows.  Every output is the same chain of matrix instructions in increasing k wherever
-// its tile lies, so a row's result does not depend on the rows beside it.  K, the row strides and the group
-// offsets are multiples of 8 and the operands 16-byte aligned (checked by the caller).
+// The same product for bfloat16 operands on the matrix cores (v_mfma_f32_16x16x32_bf16).
 typedef __bf16 gg_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float gg_f32x4 __attribute__((ext_vector_type(4)));
 union GGFrag {
@@ -132,157 +126,54 @@ union GGFrag {
   uint4 q;
 };
 
-// TM x TN: the tile of C a workgroup owns; its four waves lie 2 x 2 over it, each with (TM / 32) x (TN / 32) tiles of
-// 16 x 16.  Two LDS buffers: while k-step i is multiplied, the pieces of k-step i + 1 are on their way into registers
-// and go into the other buffer before the one barrier of the step.
-template <int TM, int TN, typename TC>
-__global__ void __launch_bounds__(256)
-grouped_gemm_mfma_kernel(GroupedArgs p) {
-  constexpr int MT = TM / 32, NT = TN / 32;          // 16-row / 16-column tiles a wave
-  constexpr int PA = TM * 4 / 256, PW = TN * 4 / 256;  // 16-byte pieces of A / W a thread brings in per k-step
-  __shared__ uint4 As[2][TM * 4];
-  __shared__ uint4 Ws[2][TN * 4];
-  __shared__ int a_rows[TM];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int n0 = blockIdx.x * TN;
-  int g, m0, m_end, c_row0;
-  if (p.offs) {
-    int tile = blockIdx.y, start = 0, cnt = 0;
-    for (g = 0; g < p.G; ++g) {
-      start = p.offs[g];
-      cnt = p.offs[g + 1] - start;
-      const int nt = (cnt + TM - 1) / TM;
-      if (tile < nt) break;
-      tile -= nt;
-    }
-    if (g == p.G) return;
-    m0 = tile * TM;
-    m_end = cnt;
-    c_row0 = start;
-    for (int i = tid; i < TM; i += 256) {
-      const int r = m0 + i;
-      a_rows[i] = r < cnt ? (p.gather ? p.gather[start + r] / p.gather_div : start + r) : -1;
-    }
-  } else {
-    g = blockIdx.z;
-    m0 = blockIdx.y * TM;
-    m_end = p.M;
-    c_row0 = 0;
-    for (int i = tid; i < TM; i += 256) a_rows[i] = m0 + i < p.M ? m0 + i : -1;
-  }
-  __syncthreads();
-  const bf16* A = (const bf16*)p.A + (size_t)(g % p.a_mod) * p.a_group;
-  const bf16* W = (const bf16*)p.W + (size_t)g * p.w_group;
-  // piece j of this thread: row (tid + 256 j) / 4, k-block tid % 4
-  const int lkb = tid & 3;
-  const bf16* a_src[PA];
-  const bf16* w_src[PW];
-  int a_put[PA], w_put[PW];
-#pragma unroll
-  for (int j = 0; j < PA; ++j) {
-    const int row = (tid >> 2) + 64 * j, ar = a_rows[row];
-    a_src[j] = ar >= 0 ? A + (size_t)ar * p.lda + lkb * 8 : nullptr;
-    a_put[j] = row * 4 + (lkb ^ ((row >> 2) & 3));
-  }
-#pragma unroll
-  for (int j = 0; j < PW; ++j) {
-    const int row = (tid >> 2) + 64 * j;
-    w_src[j] = n0 + row < p.N ? W + (size_t)(n0 + row) * p.ldw + lkb * 8 : nullptr;
-    w_put[j] = row * 4 + (lkb ^ ((row >> 2) & 3));
-  }
-  const uint4 zero = make_uint4(0, 0, 0, 0);
-  auto fetch = [&](const bf16* src, int k0) { return src && k0 + lkb * 8 < p.K ? *reinterpret_cast<const uint4*>(src + k0) : zero; };
-  const int col = lane & 15, kb = lane >> 4;
-  const int wm = (wave >> 1) * (TM / 2), wn = (wave & 1) * (TN / 2);
-  gg_f32x4 acc[MT][NT];
-#pragma unroll
-  for (int i = 0; i < MT; ++i)
-#pragma unroll
-    for (int j = 0; j < NT; ++j) acc[i][j] = gg_f32x4{0.f, 0.f, 0.f, 0.f};
-  uint4 ra[PA], rw[PW];
-#pragma unroll
-  for (int j = 0; j < PA; ++j) As[0][a_put[j]] = fetch(a_src[j], 0);
-#pragma unroll
-  for (int j = 0; j < PW; ++j) Ws[0][w_put[j]] = fetch(w_src[j], 0);
-  __syncthreads();
-  int cur = 0;
-  for (int k0 = 0; k0 < p.K; k0 += 32) {
-    const bool more = k0 + 32 < p.K;
-    if (more) {
-#pragma unroll
-      for (int j = 0; j < PA; ++j) ra[j] = fetch(a_src[j], k0 + 32);
-#pragma unroll
-      for (int j = 0; j < PW; ++j) rw[j] = fetch(w_src[j], k0 + 32);
-    }
-    GGFrag a[MT], b[NT];
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      const int r = wm + i * 16 + col;
-      a[i].q = As[cur][r * 4 + (kb ^ ((r >> 2) & 3))];
-    }
-#pragma unroll
-    for (int j = 0; j < NT; ++j) {
-      const int r = wn + j * 16 + col;
-      b[j].q = Ws[cur][r * 4 + (kb ^ ((r >> 2) & 3))];
-    }
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int j = 0; j < NT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[j].v, acc[i][j], 0, 0, 0);
-    if (more) {
-#pragma unroll
-      for (int j = 0; j < PA; ++j) As[cur ^ 1][a_put[j]] = ra[j];
-#pragma unroll
-      for (int j = 0; j < PW; ++j) Ws[cur ^ 1][w_put[j]] = rw[j];
-    }
-    __syncthreads();
-    cur ^= 1;
-  }
-  TC* C = (TC*)p.C + (size_t)g * p.c_group;
-#pragma unroll
-  for (int j = 0; j < NT; ++j) {
-    const int n = n0 + wn + j * 16 + col;
-    if (n >= p.N) continue;
-    const float bias = p.bias ? p.bias[(size_t)g * p.N + n] : 0.f;
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int m = m0 + wm + i * 16 + kb * 4 + e;
-        if (m >= m_end) continue;
-        const size_t crow = (size_t)(c_row0 + m);
-        float v = mie_act(acc[i][j][e] + bias, p.act);
-        if (p.gate) v *= mie_sigmoid(p.gate[crow * p.ldg + (size_t)g * p.N + n]);
-        C[crow * p.ldc + n] = from_float<TC>(v);
-      }
-  }
-}
-
-// Tiles of 128 x 128 for steps of many rows: the k-steps come into a ring of three LDS stages by loads that write the
-// LDS directly (no registers in between, two stages on their way while the third is multiplied), 1 KB a fragment of
-// 16 rows x 32 k: lane l brings k-block (l % 4) ^ (l / 16) % 4 of row l / 4, which is the slot order above.  A lane
-// whose row or k-block does not exist reads from a block of zeros instead, so every wave issues the same four loads a
-// stage and one count tells when a stage has landed.  The fragments are read back in one piece of assembly with its
-// own wait: the compiler does not know of the loads that write the LDS.
+// A workgroup of four waves (2 x 2) owns TM x 128 of C.  The k-steps of 32 come into a ring of LDS stages by loads that
+// write the LDS directly (no registers in between; all stages but one are on their way while one is multiplied),
+// 1 KB a fragment of 16 rows x 32 k: lane l brings k-block (l % 4) ^ (l / 16) % 4 of row l / 4, so that the piece of
+// row r, k-block b sits at slot 4 r + (b ^ (r / 4) % 4) and the fragment reads spread over all banks.  A lane whose row
+// or k-block does not exist reads from a block of zeros instead, so every wave issues the same loads a stage and one
+// count tells when a stage has landed.  The fragments are read back in one piece of assembly with its own wait: the
+// compiler does not know of the loads that write the LDS.  TM = 128 with three stages for steps of many rows; TM = 64
+// with five stages for few rows (decode steps: the weights stream, and what counts is the bytes on their way).
+// Every output is the same chain of matrix instructions in increasing k wherever its tile lies, so a row's result
+// does not depend on the rows beside it.  K, the row strides and the group offsets are multiples of 8 and the
+// operands 16-byte aligned (checked by the caller).
 #define GG_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
 typedef uint32_t gg_u32x4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ void gg_read4(uint32_t base, gg_u32x4 (&f)[4]) {
-  asm volatile(
-    "ds_read_b128 %0, %4\n\t"
-    "ds_read_b128 %1, %4 offset:1024\n\t"
-    "ds_read_b128 %2, %4 offset:2048\n\t"
-    "ds_read_b128 %3, %4 offset:3072\n\t"
-    "s_waitcnt lgkmcnt(0)"
-    : "=&v"(f[0]), "=&v"(f[1]), "=&v"(f[2]), "=&v"(f[3])
-    : "v"(base)
-    : "memory");
-}
+template <int N> struct GGRead;
+template <> struct GGRead<4> {
+  static __device__ __forceinline__ void run(uint32_t base, gg_u32x4 (&f)[4]) {
+    asm volatile(
+      "ds_read_b128 %0, %4\n\t"
+      "ds_read_b128 %1, %4 offset:1024\n\t"
+      "ds_read_b128 %2, %4 offset:2048\n\t"
+      "ds_read_b128 %3, %4 offset:3072\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(f[0]), "=&v"(f[1]), "=&v"(f[2]), "=&v"(f[3])
+      : "v"(base)
+      : "memory");
+  }
+};
+template <> struct GGRead<2> {
+  static __device__ __forceinline__ void run(uint32_t base, gg_u32x4 (&f)[2]) {
+    asm volatile(
+      "ds_read_b128 %0, %2\n\t"
+      "ds_read_b128 %1, %2 offset:1024\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(f[0]), "=&v"(f[1])
+      : "v"(base)
+      : "memory");
+  }
+};
 
-template <typename TC>
+template <int TM, int STAGES, typename TC>
 __global__ void __launch_bounds__(256)
 grouped_gemm_ring_kernel(GroupedArgs p) {
-  constexpr int TM = 128, TN = 128, STAGES = 3, STAGE_BYTES = (TM + TN) * 64;
+  constexpr int TN = 128, FA = TM / 16, FW = TN / 16, LPW = (FA + FW) / 4, MT = TM / 32, NT = 4;
+  constexpr int STAGE_BYTES = (FA + FW) * 1024;
+  static_assert((FA + FW) % 4 == 0, "the fragments of a stage must divide over the waves");
+  static_assert(STAGES * STAGE_BYTES + TM * 4 <= 65536, "LDS");
+  static_assert(LPW * (STAGES - 2) <= 63, "more loads in flight than the counter holds");
   __shared__ __align__(16) char lds[STAGES * STAGE_BYTES];
   __shared__ int a_rows[TM];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -315,53 +206,56 @@ grouped_gemm_ring_kernel(GroupedArgs p) {
   __syncthreads();
   const bf16* A = (const bf16*)p.A + (size_t)(g % p.a_mod) * p.a_group;
   const bf16* W = (const bf16*)p.W + (size_t)g * p.w_group;
-  // what this lane brings in: fragments 2 wave and 2 wave + 1 of A and of W, row lane / 4 of each
+  // what this lane brings in: row lane / 4 of the fragments wave * LPW .. (A's fragments come first in a stage)
   const int lrow = lane >> 2, lkb = (lane & 3) ^ ((lane >> 4) & 3);
   const bf16* zero_lane = (const bf16*)p.zeros + lkb * 8;
-  const bf16* src[4];
+  const bf16* src[LPW];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int ar = a_rows[(2 * wave + j) * 16 + lrow];
-    src[j] = ar >= 0 ? A + (size_t)ar * p.lda + lkb * 8 : nullptr;
-    const int n = n0 + (2 * wave + j) * 16 + lrow;
-    src[2 + j] = n < p.N ? W + (size_t)n * p.ldw + lkb * 8 : nullptr;
+  for (int j = 0; j < LPW; ++j) {
+    const int f = wave * LPW + j;
+    if (f < FA) {
+      const int ar = a_rows[f * 16 + lrow];
+      src[j] = ar >= 0 ? A + (size_t)ar * p.lda + lkb * 8 : nullptr;
+    } else {
+      const int n = n0 + (f - FA) * 16 + lrow;
+      src[j] = n < p.N ? W + (size_t)n * p.ldw + lkb * 8 : nullptr;
+    }
   }
   auto issue = [&](int s) {
-    char* base = lds + (s % STAGES) * STAGE_BYTES;
+    char* base = lds + (s % STAGES) * STAGE_BYTES + wave * LPW * 1024;
     const int k0 = s * 32;
     const bool kok = k0 + lkb * 8 < p.K;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < LPW; ++j) {
       const bf16* from = src[j] && kok ? src[j] + k0 : zero_lane;
-      const int frag = (j < 2 ? 0 : TM / 16) + 2 * wave + (j & 1);
       __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)from,
-                                       (__attribute__((address_space(3))) void*)(base + frag * 1024), 16, 0, 0);
+                                       (__attribute__((address_space(3))) void*)(base + j * 1024), 16, 0, 0);
     }
   };
   const int col = lane & 15, kb = lane >> 4;
   const int rslot = col * 4 + (kb ^ ((col >> 2) & 3));
   const uint32_t lds0 = (uint32_t)(size_t)(__attribute__((address_space(3))) char*)lds;
-  const uint32_t a_off = (wave >> 1) * 4096 + rslot * 16, b_off = TM * 64 + (wave & 1) * 4096 + rslot * 16;
-  gg_f32x4 acc[4][4];
+  const uint32_t a_off = (wave >> 1) * MT * 1024 + rslot * 16, b_off = FA * 1024 + (wave & 1) * NT * 1024 + rslot * 16;
+  gg_f32x4 acc[MT][NT];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = gg_f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < NT; ++j) acc[i][j] = gg_f32x4{0.f, 0.f, 0.f, 0.f};
   const int nk = (p.K + 31) / 32;
-  issue(0);
-  issue(1);
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) issue(s);
   for (int it = 0; it < nk; ++it) {
-    GG_VMCNT(4);                       // this wave's loads of stage `it` have landed
+    GG_VMCNT(LPW * (STAGES - 2));      // this wave's loads of stage `it` have landed
     __builtin_amdgcn_s_barrier();      // and everybody else's; everybody is done reading stage it - 1
-    issue(it + 2);                     // into the buffer stage it - 1 used (zeros beyond K)
+    issue(it + STAGES - 1);            // into the buffer stage it - 1 used (zeros beyond K)
     const uint32_t base = lds0 + (it % STAGES) * STAGE_BYTES;
-    gg_u32x4 fa[4], fb[4];
-    gg_read4(base + a_off, fa);
-    gg_read4(base + b_off, fb);
+    gg_u32x4 fa[MT], fb[NT];
+    GGRead<MT>::run(base + a_off, fa);
+    GGRead<NT>::run(base + b_off, fb);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MT; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
+      for (int j = 0; j < NT; ++j) {
         GGFrag a, b;
         a.q = *reinterpret_cast<uint4*>(&fa[i]);
         b.q = *reinterpret_cast<uint4*>(&fb[j]);
@@ -369,15 +263,15 @@ grouped_gemm_ring_kernel(GroupedArgs p) {
       }
   }
   GG_VMCNT(0);                         // nothing of this wave may still be writing the LDS when it ends
-  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+  const int wm = (wave >> 1) * (TM / 2), wn = (wave & 1) * (TN / 2);
   TC* C = (TC*)p.C + (size_t)g * p.c_group;
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < NT; ++j) {
     const int n = n0 + wn + j * 16 + col;
     if (n >= p.N) continue;
     const float bias = p.bias ? p.bias[(size_t)g * p.N + n] : 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < MT; ++i)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int m = m0 + wm + i * 16 + kb * 4 + e;
@@ -423,21 +317,21 @@ MIE_EXPORT int mie_grouped_linear(const void* A, int a_dtype, long lda, long a_g
   const long mt = (M + GG_T - 1) / GG_T + (offs ? G : 0);
   if (mt > 65535 || G > 65535) MIE_FAIL("grouped_linear: %ld row tiles, %d groups are beyond the grid", mt, G);
   dim3 grid((N + GG_T - 1) / GG_T, (unsigned)mt, offs ? 1 : G);
-  // bfloat16 operands that the matrix-core kernel's 16-byte loads can take: tiles of 128 x 128 where there are rows
-  // enough to fill them (a function of the step's size, not of a row's place in it), of 64 x 64 otherwise
-  if (a_dtype == MIE_BF16 && w_dtype == MIE_BF16 && (c_dtype == MIE_BF16 || c_dtype == MIE_F32) && K % 8 == 0 && lda % 8 == 0 &&
-      ldw % 8 == 0 && p.a_group % 8 == 0 && w_group % 8 == 0 && (((uintptr_t)A | (uintptr_t)W) & 15) == 0) {
-    const bool big = zeros && (offs ? M >= 128L * G : M >= 256);
+  // bfloat16 operands that the matrix-core kernel's 16-byte loads can take: row tiles of 128 where there are rows
+  // enough to fill them (a function of the step's size, not of a row's place in it), of 64 otherwise
+  if (zeros && a_dtype == MIE_BF16 && w_dtype == MIE_BF16 && (c_dtype == MIE_BF16 || c_dtype == MIE_F32) && K % 8 == 0 &&
+      lda % 8 == 0 && ldw % 8 == 0 && p.a_group % 8 == 0 && w_group % 8 == 0 && (((uintptr_t)A | (uintptr_t)W) & 15) == 0) {
+    const bool big = offs ? M >= 128L * G : M >= 256;
     const int T = big ? 128 : 64;
     const long mtiles = (M + T - 1) / T + (offs ? G : 0);
     if (mtiles > 65535) MIE_FAIL("grouped_linear: %ld row tiles are beyond the grid", mtiles);
-    dim3 mgrid((N + T - 1) / T, (unsigned)mtiles, offs ? 1 : G);
-#define GG_MFMA(T_, TC_) hipLaunchKernelGGL((grouped_gemm_mfma_kernel<T_, T_, TC_>), mgrid, dim3(256), 0, s, p)
-    if (big && c_dtype == MIE_BF16) hipLaunchKernelGGL(grouped_gemm_ring_kernel<bf16>, mgrid, dim3(256), 0, s, p);
-    else if (big) hipLaunchKernelGGL(grouped_gemm_ring_kernel<float>, mgrid, dim3(256), 0, s, p);
-    else if (c_dtype == MIE_BF16) GG_MFMA(64, bf16);
-    else GG_MFMA(64, float);
-#undef GG_MFMA
+    dim3 mgrid((N + 127) / 128, (unsigned)mtiles, offs ? 1 : G);
+#define GG_RING(TM_, ST_, TC_) hipLaunchKernelGGL((grouped_gemm_ring_kernel<TM_, ST_, TC_>), mgrid, dim3(256), 0, s, p)
+    if (big && c_dtype == MIE_BF16) GG_RING(128, 3, bf16);
+    else if (big) GG_RING(128, 3, float);
+    else if (c_dtype == MIE_BF16) GG_RING(64, 5, bf16);
+    else GG_RING(64, 5, float);
+#undef GG_RING
     MIE_CHECK_LAUNCH("grouped_linear");
     return 0;
   }
