@@ -118,6 +118,41 @@ grouped_gemm_kernel(GroupedArgs p) {
   }
 }
 
+// Few rows (a decode step) in the columns shape, any operand types, 32-bit FMAs: one wave an output column, the lanes
+// spread over k (a weight row is read once, 64 consecutive numbers at a time), every lane one partial sum a row, then
+// the wave's sum.  The order of a sum depends on K alone.
+#define GV_ROWS 16
+template <typename TA, typename TW, typename TC>
+__global__ void __launch_bounds__(256)
+grouped_gemv_kernel(GroupedArgs p) {
+  const int lane = threadIdx.x & 63;
+  const int n = blockIdx.x * 4 + (threadIdx.x >> 6), g = blockIdx.z;
+  if (n >= p.N) return;
+  const TA* A = (const TA*)p.A + (size_t)(g % p.a_mod) * p.a_group;
+  const TW* w = (const TW*)p.W + (size_t)g * p.w_group + (size_t)n * p.ldw;
+  float acc[GV_ROWS];
+#pragma unroll
+  for (int m = 0; m < GV_ROWS; ++m) acc[m] = 0.f;
+  for (int k = lane; k < p.K; k += 64) {
+    const float wv = to_float(w[k]);
+#pragma unroll
+    for (int m = 0; m < GV_ROWS; ++m)
+      if (m < p.M) acc[m] = fmaf(to_float(A[(size_t)m * p.lda + k]), wv, acc[m]);
+  }
+  TC* C = (TC*)p.C + (size_t)g * p.c_group;
+  const float bias = p.bias ? p.bias[(size_t)g * p.N + n] : 0.f;
+#pragma unroll
+  for (int m = 0; m < GV_ROWS; ++m) {
+    if (m >= p.M) break;
+    float v = wave_sum(acc[m]);
+    if (lane == 0) {
+      v = mie_act(v + bias, p.act);
+      if (p.gate) v *= mie_sigmoid(p.gate[(size_t)m * p.ldg + (size_t)g * p.N + n]);
+      C[(size_t)m * p.ldc + n] = from_float<TC>(v);
+    }
+  }
+}
+
 // The same product for bfloat16 operands on the matrix cores (v_mfma_f32_16x16x32_bf16).
 typedef __bf16 gg_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float gg_f32x4 __attribute__((ext_vector_type(4)));
@@ -288,6 +323,15 @@ MIE_EXPORT const char* grouped_gemm_last_error() { return g_mie_error; }
 
 template <typename TA, typename TW>
 static int launch_grouped(const GroupedArgs& p, int c_dtype, dim3 grid, hipStream_t s) {
+  if (!p.offs && p.M <= GV_ROWS && (c_dtype == MIE_F32 || c_dtype == MIE_BF16)) {     // few rows: a wave a column
+    dim3 vgrid((p.N + 3) / 4, 1, p.G);
+    if (c_dtype == MIE_F32)
+      hipLaunchKernelGGL((grouped_gemv_kernel<TA, TW, float>), vgrid, dim3(256), 0, s, p);
+    else
+      hipLaunchKernelGGL((grouped_gemv_kernel<TA, TW, bf16>), vgrid, dim3(256), 0, s, p);
+    MIE_CHECK_LAUNCH("grouped_linear");
+    return 0;
+  }
   if (c_dtype == MIE_F32)
     hipLaunchKernelGGL((grouped_gemm_kernel<TA, TW, float>), grid, dim3(256), 0, s, p);
   else if (c_dtype == MIE_BF16)
