@@ -73,7 +73,9 @@ template <int SLOTS, int IT> struct RingStart {
   }
 };
 
-enum { EPI_STORE_BF16 = 0, EPI_STORE_F32 = 1, EPI_ADD = 2, EPI_SWIGLU = 3, EPI_ROPE = 4 };
+enum { EPI_STORE_BF16 = 0, EPI_STORE_F32 = 1, EPI_ADD = 2, EPI_SWIGLU = 3, EPI_ROPE = 4, EPI_GEGLU = 5 };
+// the gated epilogues differ in the gate's function only: silu (SWIGLU) or the tanh form of gelu (GEGLU)
+#define EPI_GATED(E) ((E) == EPI_SWIGLU || (E) == EPI_GEGLU)
 
 // What the rotary epilogue needs beside the product: W is the fused q/k/v projection; the workgroup owns
 // columns j0 .. j0 + 7 and j0 + D/2 .. j0 + D/2 + 7 of one head, i.e. 8 rotary pairs.
@@ -113,7 +115,7 @@ struct NormArgs {
 // so that both members of a pair are lanes c and c ^ 8 of one wave after the reduction.
 template <int EPI>
 __device__ __forceinline__ long tile_column(int tile, int c, int N, int up_offset, int D, bool& ok) {
-  if (EPI == EPI_SWIGLU) {
+  if (EPI_GATED(EPI)) {
     const int j = tile * 8 + (c & 7);
     ok = j < N;
     return (long)(c >> 3) * up_offset + j;
@@ -296,7 +298,7 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
   const float rstd = NF ? s_rstd[m] : 1.f;
   const float mine_v = v * rstd;
   float other = 0.f;
-  if (EPI == EPI_ROPE || EPI == EPI_SWIGLU) other = __shfl_xor(mine_v, 8, 64);   // the pair's other member
+  if (EPI == EPI_ROPE || EPI_GATED(EPI)) other = __shfl_xor(mine_v, 8, 64);   // the pair's other member
   if (!live) return;
   if (EPI == EPI_ROPE) {
     const int D = rope.D;
@@ -318,8 +320,9 @@ skinny_gemm_kernel(const bf16* __restrict__ X, long ldx, const bf16* __restrict_
     ((bf16*)outv)[(size_t)m * ldo + n] = __float2bfloat16(mine_v);
   } else if (EPI == EPI_STORE_F32) {
     ((float*)outv)[(size_t)m * ldo + n] = mine_v;
-  } else if (c < 8) {                        // SWIGLU: mine = gate, other = up
-    ((bf16*)outv)[(size_t)m * ldo + n] = __float2bfloat16(mine_v / (1.0f + expf(-mine_v)) * other);
+  } else if (c < 8) {                        // gated: mine = gate, other = up
+    const float a = EPI == EPI_GEGLU ? mie_gelu_tanh(mine_v) : mine_v / (1.0f + expf(-mine_v));
+    ((bf16*)outv)[(size_t)m * ldo + n] = __float2bfloat16(a * other);
   }
 }
 
@@ -355,6 +358,7 @@ static int launch_epi(int epi, dim3 grid, hipStream_t s, const bf16* X, long ldx
     case EPI_STORE_F32: SG_LAUNCH(EPI_STORE_F32); break;
     case EPI_ADD: SG_LAUNCH(EPI_ADD); break;
     case EPI_SWIGLU: SG_LAUNCH(EPI_SWIGLU); break;
+    case EPI_GEGLU: SG_LAUNCH(EPI_GEGLU); break;
     case EPI_ROPE: SG_LAUNCH(EPI_ROPE); break;
     default: MIE_FAIL("skinny_gemm: epilogue code %d", epi);
   }
@@ -421,13 +425,13 @@ static int fill_norm_args(NormArgs& nf, int epi, const void* next_g, int next_g_
 }
 
 // X [M, K] and W bfloat16.  epi: 0 bfloat16 y, 1 float32 y, 2 out[m, n] += y (float32), 3 silu(gate) * up with
-// W = [gate rows (N of them); up rows] and N = the intermediate size.
+// W = [gate rows (N of them); up rows] and N = the intermediate size, 5 the same with gelu_tanh(gate).
 MIE_EXPORT int mie_skinny_gemm(const void* X, long ldx, const void* W, long ldw, void* out, long ldo, int epi, int M,
                                int N, int K, const void* next_g, int next_g_f32, void* x_next, long ldx_next,
                                float* ss_out, const float* ss_in, int ss_tiles, float eps, const int* rows,
                                hipStream_t s) {
   if (M <= 0 || N <= 0) return 0;
-  if (epi < 0 || epi > EPI_SWIGLU) MIE_FAIL("skinny_gemm: epilogue code %d", epi);
+  if (epi < 0 || (epi > EPI_SWIGLU && epi != EPI_GEGLU)) MIE_FAIL("skinny_gemm: epilogue code %d", epi);
   if (check_operands("skinny_gemm", X, ldx, W, ldw, M, K)) return -1;
   if (ldo < N) MIE_FAIL("skinny_gemm: output leading dim %ld < %d", ldo, N);
   RopeArgs none = {};
@@ -435,7 +439,7 @@ MIE_EXPORT int mie_skinny_gemm(const void* X, long ldx, const void* W, long ldw,
   const bool fused = next_g || ss_in;
   if (fused && fill_norm_args(nf, epi, next_g, next_g_f32, x_next, ldx_next, ss_out, ss_in, ss_tiles, K, eps, rows, N)) return -1;
   if (!fused && rows) MIE_FAIL("skinny_gemm: a row gather comes with the fused norm only");
-  return launch_rows(epi == EPI_SWIGLU ? (N + 7) / 8 : (N + 15) / 16, epi, s, (const bf16*)X, ldx, (const bf16*)W, ldw, out, ldo, M, N, K, N, none,
+  return launch_rows(EPI_GATED(epi) ? (N + 7) / 8 : (N + 15) / 16, epi, s, (const bf16*)X, ldx, (const bf16*)W, ldw, out, ldo, M, N, K, N, none,
                      fused ? &nf : nullptr);
 }
 

@@ -200,7 +200,7 @@ class HipBackend(KernelBackend):
     # ---- few-row products of the bfloat16 path: one fused kernel each
     SKINNY_MAX_ROWS = 16      # the kernel's own limit (one tile of rows); a decode step of 16 rows of 512 keys at the
                               # benchmark's sizes takes 1.15 ms, one of 17 rows with the split product 1.27
-    EPI_BF16, EPI_F32, EPI_ADD, EPI_SWIGLU = 0, 1, 2, 3
+    EPI_BF16, EPI_F32, EPI_ADD, EPI_SWIGLU, EPI_GEGLU = 0, 1, 2, 3, 5
 
     def _skinny_ok(self, x, w, bias, rows=None) -> bool:
         """Whether the fused few-row kernel takes this product (x a bfloat16 tensor)."""
@@ -396,6 +396,12 @@ class HipBackend(KernelBackend):
             raise ValueError(f"linear_act_mul: activation {activation!r}")
         if w_gate_up.shape[0] != 2 * intermediate or x.shape[1] != w_gate_up.shape[1]:
             raise ValueError(f"linear_act_mul: x {tuple(x.shape)}, w {tuple(w_gate_up.shape)}, intermediate {intermediate}")
+        if isinstance(x, Normed):
+            x = x.materialize()
+        if activation == "gelu_tanh" and self._skinny_ok(x, w_gate_up, None):      # few rows: the gate in the product's epilogue
+            out = torch.empty((x.shape[0], intermediate), dtype=torch.bfloat16, device=w_gate_up.device)
+            self._skinny(x, w_gate_up, self.EPI_GEGLU, out, intermediate)
+            return out
         gu = self.linear(x, w_gate_up)
         out = torch.empty((gu.shape[0], intermediate), dtype=gu.dtype, device=gu.device)
         lib = self.lib("gemm")

@@ -544,3 +544,45 @@ def test_long_decoding_gpu():
                          max_model_len=208)
     got = {k: v.cpu() for k, v in trace_util.run_on_runner(runner, trace_util.decode_tail(toks, 160)).items()}
     trace_util.compare(got, expected_logits(raw, weights, toks), F32_TOL, "long decoding")
+
+
+@pytest.mark.gpu
+def test_command_line_and_trace_runner(tmp_path):
+    """The named size as a user reaches it: ``random-model`` writes the folder, ``generate`` and ``bin/trace_run``
+    load it by the architecture its config.json names; greedy tokens and replayed logits against the plain model."""
+    import os
+    import subprocess
+    import sys
+    from safetensors.torch import load_file
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    folder = str(tmp_path / "model")
+
+    def run(cmd, **kw):
+        proc = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=600, **kw)
+        assert proc.returncode == 0, f"{cmd}: exit {proc.returncode}\n{proc.stderr[-2000:]}"
+        return proc
+
+    cli = [sys.executable, "-m", "mini_inference_engine_amd"]
+    run(cli + ["random-model", "--shape", "zifelorn-tiny", "--seed", "3", "--dtype", "float32", "--out", folder])
+    raw = json.load(open(os.path.join(folder, "config.json")))
+    weights = load_file(os.path.join(folder, "model.safetensors"))
+    assert raw["architecture"] == "Zifelorn" and len(raw["layers"]) == 4
+    prompt = [5, 17, 3, 200, 41, 7, 7, 300]
+    out = run(cli + ["generate", "--model", folder, "--dtype", "float32", "--prompt-ids", ",".join(map(str, prompt)),
+                     "--max-tokens", "6", "--ignore-eos", "--quiet"])
+    rec = json.loads(out.stdout.strip().splitlines()[-1])
+    ids = list(prompt)
+    for tok in rec["output_ids"]:
+        logits = plain.forward(raw, weights, ids)[-1]
+        assert float(logits.max() - logits[tok]) <= F32_TOL * float(logits.abs().max())
+        ids.append(tok)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": ids[:9], "want": [0, 8]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": ids[9:11], "want": []}, {"id": "b", "tokens": ids[:3], "want": [2]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": ids[11:12], "want": [0]}], "end": ["a"]}]
+    out_dir = str(tmp_path / "out")
+    proc = run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", "float32", "--out", out_dir,
+                "--max-tokens", "128"], input="\n".join(json.dumps(s) for s in steps) + "\n")
+    assert [ln for ln in proc.stdout.splitlines() if ln.startswith("done")] == ["done 0", "done 1", "done 2"]
+    got = trace_util.read_outputs(out_dir, steps, raw["vocab"])
+    want = {"a": plain.forward(raw, weights, ids[:12]), "b": plain.forward(raw, weights, ids[:3])}
+    trace_util.compare(got, want, F32_TOL, "trace_run")
