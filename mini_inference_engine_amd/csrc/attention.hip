@@ -33,15 +33,15 @@ template <> struct Pack<bf16> {
   }
 };
 
-#define ATT_MAX_D 256
+#define ATT_MAX_D 1024     // head sizes up to 256 run with four accumulators a lane, larger ones with sixteen
 
-template <typename T>
+template <typename T, int NR>
 __global__ void __launch_bounds__(64)
 paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restrict__ k_cache,
                        const T* __restrict__ v_cache, T* __restrict__ out, const int* __restrict__ block_tables,
                        int max_blocks, const int* __restrict__ token_row, const int* __restrict__ positions, int Hq,
                        int Hkv, int D, int page, float scale, int window) {
-  __shared__ float qs[ATT_MAX_D];
+  __shared__ float qs[NR * 64];
   __shared__ float ps[64];
   __shared__ long long base[64];     // per key of the chunk: offset of its value column
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
@@ -55,9 +55,9 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
 
   typedef Pack<T> P;
   float m = -INFINITY, l = 0.f;
-  float acc[ATT_MAX_D / 64];
+  float acc[NR];
 #pragma unroll
-  for (int i = 0; i < ATT_MAX_D / 64; ++i) acc[i] = 0.f;
+  for (int i = 0; i < NR; ++i) acc[i] = 0.f;
 
   for (int c0 = lo; c0 <= pos; c0 += 64) {
     const int key = c0 + lane;
@@ -85,12 +85,12 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
     __syncthreads();
     const int nk = pos - c0 + 1 < 64 ? pos - c0 + 1 : 64;
 #pragma unroll
-    for (int i = 0; i < ATT_MAX_D / 64; ++i) acc[i] *= alpha;
+    for (int i = 0; i < NR; ++i) acc[i] *= alpha;
     for (int j = 0; j < nk; ++j) {
       const float pj = ps[j];
       const T* vp = v_cache + base[j];
 #pragma unroll
-      for (int i = 0; i < ATT_MAX_D / 64; ++i) {
+      for (int i = 0; i < NR; ++i) {
         const int d = lane + 64 * i;
         if (d < D) acc[i] = fmaf(pj, to_float(vp[(size_t)d * page]), acc[i]);
       }
@@ -101,7 +101,7 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
   const float inv = 1.0f / l;
   T* op = out + ((size_t)t * Hq + h) * D;
 #pragma unroll
-  for (int i = 0; i < ATT_MAX_D / 64; ++i) {
+  for (int i = 0; i < NR; ++i) {
     const int d = lane + 64 * i;
     if (d < D) op[d] = from_float<T>(acc[i] * inv);
   }
@@ -120,16 +120,16 @@ MIE_EXPORT int mie_paged_attention(const void* q, long q_stride, const void* k_c
   if (page <= 0 || max_blocks <= 0) MIE_FAIL("paged_attention: page %d, max_blocks %d", page, max_blocks);
   if (q_stride < (long)Hq * D) MIE_FAIL("paged_attention: q row stride %ld < %d", q_stride, Hq * D);
   dim3 grid(tokens, Hq), block(64);
-  if (dtype == MIE_F32)
-    hipLaunchKernelGGL(paged_attention_kernel<float>, grid, block, 0, stream, (const float*)q, q_stride,
-                       (const float*)k_cache, (const float*)v_cache, (float*)out, block_tables, max_blocks, token_row,
-                       positions, Hq, Hkv, D, page, scale, window);
-  else if (dtype == MIE_BF16)
-    hipLaunchKernelGGL(paged_attention_kernel<bf16>, grid, block, 0, stream, (const bf16*)q, q_stride,
-                       (const bf16*)k_cache, (const bf16*)v_cache, (bf16*)out, block_tables, max_blocks, token_row,
-                       positions, Hq, Hkv, D, page, scale, window);
-  else
-    MIE_FAIL("paged_attention: dtype code %d", dtype);
+#define PA_LAUNCH(T_, NR_)                                                                                               \
+  hipLaunchKernelGGL((paged_attention_kernel<T_, NR_>), grid, block, 0, stream, (const T_*)q, q_stride, (const T_*)k_cache, \
+                     (const T_*)v_cache, (T_*)out, block_tables, max_blocks, token_row, positions, Hq, Hkv, D, page, scale,  \
+                     window)
+  if (dtype == MIE_F32 && D <= 256) PA_LAUNCH(float, 4);
+  else if (dtype == MIE_F32) PA_LAUNCH(float, 16);
+  else if (dtype == MIE_BF16 && D <= 256) PA_LAUNCH(bf16, 4);
+  else if (dtype == MIE_BF16) PA_LAUNCH(bf16, 16);
+  else MIE_FAIL("paged_attention: dtype code %d", dtype);
+#undef PA_LAUNCH
   MIE_CHECK_LAUNCH("paged_attention");
   return 0;
 }

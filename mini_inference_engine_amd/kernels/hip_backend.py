@@ -868,6 +868,8 @@ class HipBackend(KernelBackend):
         T, page, bt = self._check_attention(qkv, Hq, Hkv, D, k_cache, v_cache, group, step)
         out = torch.empty((T, Hq * D), dtype=qkv.dtype, device=qkv.device)
         done = 0
+        if D > 256:
+            force_generic = True            # beyond the matrix-core kernels' head sizes: the 32-bit kernel takes up to 1,024
         if qkv.dtype == torch.bfloat16 and not force_generic and step.num_decode_rows > 0:
             done = step.num_decode_rows        # single-token rows lead the batch: token t is row t
             lib = self.lib("attention_bf16", (f"-DHEAD_DIM={D}",))

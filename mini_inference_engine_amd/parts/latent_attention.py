@@ -49,7 +49,7 @@ class PagedLatent(CacheRequirement):
 
 @register_mixer("latent_attention")
 class LatentAttention(Mixer):
-    MAX_PADDED_DIM = 256        # what the attention kernels take as a head size
+    MAX_PADDED_DIM = 1024       # what the attention kernels take as a head size (the matrix-core ones up to 256)
 
     def __init__(self, width: int, num_heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, q_rank: int,
                  scale: float, eps: float, position, prefix: str, has_kv: bool = True, gated: bool = True,

@@ -586,3 +586,19 @@ def test_command_line_and_trace_runner(tmp_path):
     got = trace_util.read_outputs(out_dir, steps, raw["vocab"])
     want = {"a": plain.forward(raw, weights, ids[:12]), "b": plain.forward(raw, weights, ids[:3])}
     trace_util.compare(got, want, F32_TOL, "trace_run")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_latent_wider_than_the_matrix_core_kernels_gpu(dtype):
+    """kv_rank + rot_dim = 288 numbers a token: beyond the head sizes of the matrix-core attention kernels, so both
+    dtypes run the 32-bit attention kernel; a portion, single tokens and a second request beside it."""
+    raw = one_layer("latent_attention", att(2, 16, 16, 16, 272, 32), dict(kind="dense", ff=48), width=64, vocab=90)
+    cfg = ZifelornConfig.from_dict(raw)
+    weights = random_tensors(cfg, 8, torch.float32, std=0.2)
+    weights = {k: v.to(torch.float32 if dtype == "float32" else torch.bfloat16) for k, v in weights.items()}
+    prompts = trace_util.random_prompts(90, [50, 21], seed=1)
+    runner = ModelRunner(cfg, weights=weights, dtype=dtype, num_pages=12, max_rows=2, max_step_tokens=64, max_model_len=128)
+    got = {k: v.cpu() for k, v in trace_util.run_on_runner(runner, trace_util.mixed(prompts, 2, seed=2, tail=5)).items()}
+    check = trace_util.compare if dtype == "float32" else compare_most
+    check(got, expected_logits(raw, weights, prompts), F32_TOL if dtype == "float32" else BF16_TOL_PER_LAYER, f"wide latent {dtype}")
