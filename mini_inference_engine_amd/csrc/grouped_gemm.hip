@@ -167,7 +167,7 @@ union GGFrag {
 // row r, k-block b sits at slot 4 r + (b ^ (r / 4) % 4) and the fragment reads spread over all banks.  A lane whose row
 // or k-block does not exist reads from a block of zeros instead, so every wave issues the same loads a stage and one
 // count tells when a stage has landed.  The fragments are read back in one piece of assembly with its own wait: the
-// compiler does not know of the loads that write the LDS.  TM = 128 with three stages for steps of many rows; TM = 64
+// compiler does not know of the loads that write the LDS.  TM = 128 with three stages for steps of many rows (four were measured: no faster); TM = 64
 // with five stages for few rows (decode steps: the weights stream, and what counts is the bytes on their way).
 // Every output is the same chain of matrix instructions in increasing k wherever its tile lies, so a row's result
 // does not depend on the rows beside it.  K, the row strides and the group offsets are multiples of 8 and the
@@ -207,10 +207,9 @@ grouped_gemm_ring_kernel(GroupedArgs p) {
   constexpr int TN = 128, FA = TM / 16, FW = TN / 16, LPW = (FA + FW) / 4, MT = TM / 32, NT = 4;
   constexpr int STAGE_BYTES = (FA + FW) * 1024;
   static_assert((FA + FW) % 4 == 0, "the fragments of a stage must divide over the waves");
-  static_assert(STAGES * STAGE_BYTES + TM * 4 <= 65536, "LDS");
+  static_assert(STAGES * STAGE_BYTES <= 65536, "LDS");
   static_assert(LPW * (STAGES - 2) <= 63, "more loads in flight than the counter holds");
   __shared__ __align__(16) char lds[STAGES * STAGE_BYTES];
-  __shared__ int a_rows[TM];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int n0 = blockIdx.x * TN;
   int g, m0, m_end, c_row0;
@@ -227,18 +226,12 @@ grouped_gemm_ring_kernel(GroupedArgs p) {
     m0 = tile * TM;
     m_end = cnt;
     c_row0 = start;
-    if (tid < TM) {
-      const int r = m0 + tid;
-      a_rows[tid] = r < cnt ? (p.gather ? p.gather[start + r] / p.gather_div : start + r) : -1;
-    }
   } else {
     g = blockIdx.z;
     m0 = blockIdx.y * TM;
     m_end = p.M;
     c_row0 = 0;
-    if (tid < TM) a_rows[tid] = m0 + tid < p.M ? m0 + tid : -1;
   }
-  __syncthreads();
   const bf16* A = (const bf16*)p.A + (size_t)(g % p.a_mod) * p.a_group;
   const bf16* W = (const bf16*)p.W + (size_t)g * p.w_group;
   // what this lane brings in: row lane / 4 of the fragments wave * LPW .. (A's fragments come first in a stage)
@@ -249,7 +242,8 @@ grouped_gemm_ring_kernel(GroupedArgs p) {
   for (int j = 0; j < LPW; ++j) {
     const int f = wave * LPW + j;
     if (f < FA) {
-      const int ar = a_rows[f * 16 + lrow];
+      const int r = m0 + f * 16 + lrow;          // the row of the tile this lane brings in, and the row of A behind it
+      const int ar = r >= m_end ? -1 : (p.offs ? (p.gather ? p.gather[c_row0 + r] / p.gather_div : c_row0 + r) : r);
       src[j] = ar >= 0 ? A + (size_t)ar * p.lda + lkb * 8 : nullptr;
     } else {
       const int n = n0 + (f - FA) * 16 + lrow;

@@ -4,8 +4,7 @@
 //   kv_rank numbers RMS-normed (the latent c), the last rot_dim position-encoded.  The key row is [c | turned | 0],
 //   the value column [c | 0], both padded to P numbers, in the layouts the attention kernels read
 //   (keys [pages, 1, page, P], values [pages, 1, P, page]).
-// latent_query_rotate: the rotated part of every query head, turned and put behind the head's folded plain part
-//   ([T, H, P]: columns kv_rank .. kv_rank + rot_dim; the padding behind it is zeroed).
+// latent_query_rotate: the rotated part of every query head ([T, H, P]: columns kv_rank .. kv_rank + rot_dim), turned in place.
 // Rotation: elements 2i and 2i + 1 turn by the angle position * inv_freq[i], for i < n_freq; angle, cosine and sine
 // in 32-bit; elements beyond 2 n_freq pass unchanged.
 #include "common.hpp"
@@ -21,9 +20,18 @@ __global__ void __launch_bounds__(256)
 latent_kv_store_kernel(const float* __restrict__ sums, long ld, const TW* __restrict__ norm_weight, float eps,
                        const int* __restrict__ positions, const float* __restrict__ inv_freq, int n_freq,
                        TC* __restrict__ k_cache, TC* __restrict__ v_cache, const int* __restrict__ slots, int kv_rank,
-                       int rot_dim, int P, int page) {
+                       int rot_dim, int P, int page, const float* __restrict__ q_sums, const TW* __restrict__ q_weight,
+                       TC* __restrict__ q_out, int q_rank) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
+  if (q_out) {                      // the query latent of the same token, normed beside it (one kernel less a layer)
+    const float* xq = q_sums + (size_t)t * ld;
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < q_rank; i += blockDim.x) sq = fmaf(xq[i], xq[i], sq);
+    const float rq = 1.0f / sqrtf(block_sum(sq, scratch) / (float)q_rank + eps);
+    for (int i = threadIdx.x; i < q_rank; i += blockDim.x)
+      q_out[(size_t)t * q_rank + i] = from_float<TC>(xq[i] * rq * to_float(q_weight[i]));
+  }
   const float* x = sums + (size_t)t * ld;
   float ss = 0.f;
   for (int i = threadIdx.x; i < kv_rank; i += blockDim.x) ss = fmaf(x[i], x[i], ss);
@@ -50,19 +58,23 @@ latent_kv_store_kernel(const float* __restrict__ sums, long ld, const TW* __rest
 
 MIE_EXPORT const char* latent_attention_last_error() { return g_mie_error; }
 
-// sums points at the first of the kv_rank + rot_dim columns; rows are ld floats apart.
+// sums points at the first of the kv_rank + rot_dim columns; rows are ld floats apart.  q_out (or null) [tokens, q_rank] of
+// the cache's dtype: RMSNorm of the q_rank columns at q_sums (same row stride, same eps) times q_weight (the norm
+// weight's dtype).
 MIE_EXPORT int mie_latent_kv_store(const float* sums, long ld, const void* norm_weight, int w_dtype, float eps,
                                    const int* positions, const float* inv_freq, int n_freq, void* k_cache, void* v_cache,
                                    int cache_dtype, const int* slots, int tokens, int kv_rank, int rot_dim, int P, int page,
-                                   hipStream_t s) {
+                                   const float* q_sums, const void* q_weight, void* q_out, int q_rank, hipStream_t s) {
   if (tokens <= 0) return 0;
   if (kv_rank <= 0 || rot_dim < 0 || P < kv_rank + rot_dim || page <= 0 || 2 * n_freq > rot_dim)
     MIE_FAIL("latent_kv_store: kv_rank %d, rot_dim %d, padded %d, page %d, %d turned pairs", kv_rank, rot_dim, P, page, n_freq);
   if (ld < kv_rank + rot_dim || !sums || !norm_weight || !positions || !k_cache || !v_cache || !slots || (n_freq && !inv_freq))
     MIE_FAIL("latent_kv_store: operands");
+  if (q_out && (!q_sums || !q_weight || q_rank <= 0 || ld < q_rank)) MIE_FAIL("latent_kv_store: query latent operands");
 #define LKV(TW_, TC_)                                                                                                     \
   hipLaunchKernelGGL((latent_kv_store_kernel<TW_, TC_>), dim3(tokens), dim3(256), 0, s, sums, ld, (const TW_*)norm_weight, \
-                     eps, positions, inv_freq, n_freq, (TC_*)k_cache, (TC_*)v_cache, slots, kv_rank, rot_dim, P, page)
+                     eps, positions, inv_freq, n_freq, (TC_*)k_cache, (TC_*)v_cache, slots, kv_rank, rot_dim, P, page, \
+                     q_sums, (const TW_*)q_weight, (TC_*)q_out, q_rank)
   if (w_dtype == MIE_F32 && cache_dtype == MIE_F32) LKV(float, float);
   else if (w_dtype == MIE_F32 && cache_dtype == MIE_BF16) LKV(float, bf16);
   else if (w_dtype == MIE_BF16 && cache_dtype == MIE_F32) LKV(bf16, float);
@@ -73,44 +85,33 @@ MIE_EXPORT int mie_latent_kv_store(const float* sums, long ld, const void* norm_
   return 0;
 }
 
+// q [tokens, H, P] (rows ldq apart): the pairs (2i, 2i + 1), i < n_freq, of columns kv_rank .. of every head turn in place.
 template <typename T>
-__global__ void latent_query_rotate_kernel(const T* __restrict__ q, long ldq, T* __restrict__ out, const int* __restrict__ positions,
-                                           const float* __restrict__ inv_freq, int n_freq, int H, int dim, int rot_dim,
-                                           int kv_rank, int P) {
+__global__ void latent_query_rotate_kernel(T* __restrict__ q, long ldq, const int* __restrict__ positions,
+                                           const float* __restrict__ inv_freq, int n_freq, int H, int kv_rank, int P) {
   const int t = blockIdx.x, pos = positions[t];
-  const int tail = P - kv_rank;                       // columns this kernel writes in every head
-  for (int idx = threadIdx.x; idx < H * tail; idx += blockDim.x) {
-    const int h = idx / tail, j = idx - h * tail;
-    const T* src = q + (size_t)t * ldq + (size_t)h * (dim + rot_dim) + dim;
-    float v = 0.f;
-    if (j < rot_dim) {
-      const int i = j >> 1;
-      if (i < n_freq) {
-        float u0, v0;
-        turn_pair(to_float(src[2 * i]), to_float(src[2 * i + 1]), pos, inv_freq[i], u0, v0);
-        v = (j & 1) ? v0 : u0;
-      } else {
-        v = to_float(src[j]);
-      }
-    }
-    out[((size_t)t * H + h) * P + kv_rank + j] = from_float<T>(v);
+  for (int idx = threadIdx.x; idx < H * n_freq; idx += blockDim.x) {
+    const int h = idx / n_freq, i = idx - h * n_freq;
+    T* pair = q + (size_t)t * ldq + (size_t)h * P + kv_rank + 2 * i;
+    float u, v;
+    turn_pair(to_float(pair[0]), to_float(pair[1]), pos, inv_freq[i], u, v);
+    pair[0] = from_float<T>(u);
+    pair[1] = from_float<T>(v);
   }
 }
 
-// q [tokens, H (dim + rot_dim)] (row stride ldq); out [tokens, H, P] contiguous, columns kv_rank .. P of every head.
-MIE_EXPORT int mie_latent_query_rotate(const void* q, long ldq, void* out, int dtype, const int* positions,
-                                       const float* inv_freq, int n_freq, int tokens, int H, int dim, int rot_dim,
-                                       int kv_rank, int P, hipStream_t s) {
-  if (tokens <= 0 || P == kv_rank) return 0;
-  if (H <= 0 || dim <= 0 || rot_dim < 0 || P < kv_rank + rot_dim || 2 * n_freq > rot_dim || ldq < (long)H * (dim + rot_dim))
-    MIE_FAIL("latent_query_rotate: %d heads of %d + %d, padded %d, kv_rank %d", H, dim, rot_dim, P, kv_rank);
-  if (!q || !out || !positions || (n_freq && !inv_freq)) MIE_FAIL("latent_query_rotate: operands");
+MIE_EXPORT int mie_latent_query_rotate(void* q, long ldq, int dtype, const int* positions, const float* inv_freq, int n_freq,
+                                       int tokens, int H, int kv_rank, int P, hipStream_t s) {
+  if (tokens <= 0 || n_freq <= 0) return 0;
+  if (H <= 0 || kv_rank < 0 || P < kv_rank + 2 * n_freq || ldq < (long)H * P)
+    MIE_FAIL("latent_query_rotate: %d heads of %d, latent %d, %d turned pairs, row stride %ld", H, P, kv_rank, n_freq, ldq);
+  if (!q || !positions || !inv_freq) MIE_FAIL("latent_query_rotate: operands");
   if (dtype == MIE_F32)
-    hipLaunchKernelGGL(latent_query_rotate_kernel<float>, dim3(tokens), dim3(256), 0, s, (const float*)q, ldq, (float*)out,
-                       positions, inv_freq, n_freq, H, dim, rot_dim, kv_rank, P);
+    hipLaunchKernelGGL(latent_query_rotate_kernel<float>, dim3(tokens), dim3(128), 0, s, (float*)q, ldq, positions, inv_freq, n_freq,
+                       H, kv_rank, P);
   else if (dtype == MIE_BF16)
-    hipLaunchKernelGGL(latent_query_rotate_kernel<bf16>, dim3(tokens), dim3(256), 0, s, (const bf16*)q, ldq, (bf16*)out,
-                       positions, inv_freq, n_freq, H, dim, rot_dim, kv_rank, P);
+    hipLaunchKernelGGL(latent_query_rotate_kernel<bf16>, dim3(tokens), dim3(128), 0, s, (bf16*)q, ldq, positions, inv_freq, n_freq,
+                       H, kv_rank, P);
   else
     MIE_FAIL("latent_query_rotate: dtype code %d", dtype);
   MIE_CHECK_LAUNCH("latent_query_rotate");

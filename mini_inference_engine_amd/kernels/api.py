@@ -115,18 +115,19 @@ class KernelBackend:
 
     # ---- attention through a cached latent (one shared latent "head" of kv_rank + rot_dim numbers a token)
     def latent_kv_store(self, sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache,
-                        slot_mapping):
+                        slot_mapping, also_norm=None):
         """Columns [col, col + kv_rank + rot_dim) of ``sums`` [T, *] float32 are a token's down-projection.  The
         first kv_rank, RMS-normed with ``norm_weight``, are its latent c; of the last rot_dim the first
         2 * len(inv_freq) turn in adjacent pairs (2i, 2i + 1) by the angle position * inv_freq[i] (32-bit).
         Token t's slot of k_cache [pages, 1, page, P] gets [c | turned part | zeros], of v_cache [pages, 1, P, page]
-        [c | zeros] (P = the cache's padded size >= kv_rank + rot_dim)."""
+        [c | zeros] (P = the cache's padded size >= kv_rank + rot_dim).  ``also_norm`` = (col, n, weight): the same call
+        also returns rmsnorm_columns(sums, col, n, weight, eps) (the query latent beside the key/value latent)."""
         raise NotImplementedError
 
-    def latent_query(self, q, w_uk_t, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim):
-        """q [T, H (dim + rot_dim)]; w_uk_t [kv_rank, H dim], the transpose of W_uk [H dim, kv_rank].  Per head h: [q_h[:dim] W_uk,h | turned q_h[dim:] | zeros]
-        -> [T, H padded_dim] in the activation dtype: the query against a cached latent, since
-        q_h[:dim] . (W_uk,h c) = (q_h[:dim] W_uk,h) . c."""
+    def latent_query_rotate_(self, q, num_heads, kv_rank, padded_dim, positions, inv_freq):
+        """q [T, H padded_dim], every head laid out as the cache's key rows are ([against the latent | rotated part | 0]):
+        the first 2 * len(inv_freq) numbers of each head's rotated part (columns kv_rank ..) turn in place in adjacent
+        pairs by the angle position * inv_freq[i].  Returns q."""
         raise NotImplementedError
 
     def latent_value_gate(self, o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim):

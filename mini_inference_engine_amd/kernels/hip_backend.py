@@ -496,8 +496,12 @@ class HipBackend(KernelBackend):
         return page, P
 
     def latent_kv_store(self, sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache,
-                        slot_mapping):
+                        slot_mapping, also_norm=None):
         self._on_device(sums, norm_weight, positions, inv_freq, k_cache, v_cache, slot_mapping)
+        if also_norm is not None and (k_cache.dtype != self.act_dtype or also_norm[2].dtype != norm_weight.dtype):
+            # the kernel writes both in one dtype and reads both weights in one: otherwise two calls
+            self.latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache, slot_mapping)
+            return self.rmsnorm_columns(sums, also_norm[0], also_norm[1], also_norm[2], eps)
         sp = self._f32_columns(sums, col, kv_rank + rot_dim, "latent_kv_store")
         T = sums.shape[0]
         page, P = self._check_latent_cache("latent_kv_store", k_cache, v_cache, kv_rank, rot_dim)
@@ -508,29 +512,36 @@ class HipBackend(KernelBackend):
         for name, t in (("positions", positions), ("slot_mapping", slot_mapping)):
             if t.dtype != torch.int32 or t.shape[0] != T or not t.is_contiguous():
                 raise ValueError(f"latent_kv_store: {name} must be contiguous int32 [{T}]")
+        qp, qw, q_out, qn = None, None, None, 0
+        if also_norm is not None:
+            qcol, qn, qweight = also_norm
+            qp = self._f32_columns(sums, qcol, qn, "latent_kv_store: query latent")
+            if tuple(qweight.shape) != (qn,) or not qweight.is_contiguous():
+                raise ValueError(f"latent_kv_store: query norm weight {tuple(qweight.shape)} for {qn} columns")
+            self._on_device(qweight)
+            qw = _ptr(qweight)
+            q_out = torch.empty((T, qn), dtype=self.act_dtype, device=sums.device)
         lib = self.lib("latent_attention")
         library.check(lib, lib.mie_latent_kv_store(
             sp, sums.stride(0), _ptr(norm_weight), _code(norm_weight.dtype), float(eps), _ptr(positions), _ptr(inv_freq), n_freq,
-            _ptr(k_cache), _ptr(v_cache), _code(k_cache.dtype), _ptr(slot_mapping), T, kv_rank, rot_dim, P, page, self._stream()))
+            _ptr(k_cache), _ptr(v_cache), _code(k_cache.dtype), _ptr(slot_mapping), T, kv_rank, rot_dim, P, page,
+            qp, qw, _ptr(q_out), qn, self._stream()))
+        return q_out
 
-    def latent_query(self, q, w_uk_t, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim):
-        self._on_device(q, w_uk_t, positions, inv_freq)
-        _rows_ok(q, "latent_query: q")
+    def latent_query_rotate_(self, q, num_heads, kv_rank, padded_dim, positions, inv_freq):
+        self._on_device(q, positions, inv_freq)
+        _rows_ok(q, "latent_query_rotate_: q")
         H, P, T = num_heads, padded_dim, q.shape[0]
-        if q.shape[1] != H * (dim + rot_dim) or tuple(w_uk_t.shape) != (kv_rank, H * dim) or not w_uk_t.is_contiguous():
-            raise ValueError(f"latent_query: q {tuple(q.shape)}, w {tuple(w_uk_t.shape)} for {H} heads of {dim} + {rot_dim}, "
-                             f"latent {kv_rank}")
-        if P < kv_rank + rot_dim or positions.dtype != torch.int32 or positions.shape[0] != T or not positions.is_contiguous():
-            raise ValueError("latent_query: padded size or positions")
         n_freq = inv_freq.numel()
-        self._f32_vector(inv_freq, n_freq, "latent_query: inv_freq")
-        out = torch.empty((T, H * P), dtype=q.dtype, device=q.device)
-        # head h: q[:, h (dim + rot_dim) : + dim] times the columns h dim .. of the transposed W_uk -> out[:, h P : + kv_rank]
-        self._grouped(q, q.stride(0), dim + rot_dim, H, w_uk_t, H * dim, dim, out, H * P, P, T, kv_rank, dim, H)
+        if q.shape[1] != H * P or P < kv_rank + 2 * n_freq:
+            raise ValueError(f"latent_query_rotate_: q {tuple(q.shape)} for {H} heads of {P}, latent {kv_rank}, {n_freq} turned pairs")
+        if positions.dtype != torch.int32 or positions.shape[0] != T or not positions.is_contiguous():
+            raise ValueError(f"latent_query_rotate_: positions must be contiguous int32 [{T}]")
+        self._f32_vector(inv_freq, n_freq, "latent_query_rotate_: inv_freq")
         lib = self.lib("latent_attention")
-        library.check(lib, lib.mie_latent_query_rotate(_ptr(q), q.stride(0), _ptr(out), _code(q.dtype), _ptr(positions),
-                                                       _ptr(inv_freq), n_freq, T, H, dim, rot_dim, kv_rank, P, self._stream()))
-        return out
+        library.check(lib, lib.mie_latent_query_rotate(_ptr(q), q.stride(0), _code(q.dtype), _ptr(positions), _ptr(inv_freq),
+                                                       n_freq, T, H, kv_rank, P, self._stream()))
+        return q
 
     def latent_value_gate(self, o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim):
         self._on_device(o, w_uv, gate)

@@ -32,8 +32,8 @@ register_kernel_module("grouped_gemm", {
     "mie_moe_combine": [P, P, P, P, I, I, I, P],
 })
 register_kernel_module("latent_attention", {
-    "mie_latent_kv_store": [P, L, P, I, F, P, P, I, P, P, I, P, I, I, I, I, I, P],
-    "mie_latent_query_rotate": [P, L, P, I, P, P, I, I, I, I, I, I, I, P],
+    "mie_latent_kv_store": [P, L, P, I, F, P, P, I, P, P, I, P, I, I, I, I, I, P, P, P, I, P],
+    "mie_latent_query_rotate": [P, L, I, P, P, I, I, I, I, I, P],
 })
 register_kernel_module("recurrence", {
     "mie_causal_conv": [P, L, P, P, P, P, P, P, P, P, I, I, I, P],

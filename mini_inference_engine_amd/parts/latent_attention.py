@@ -6,10 +6,12 @@ W_uv,h c; queries come through a latent of their own, q = W_uq RMSNorm(W_dq x), 
 [dim plain | rot_dim rotated].  Score (q_plain . k_plain + q_rot . k_r) * scale, causal, softmax.  The
 concatenated heads are multiplied by sigmoid(W_g x) and projected by W_o.
 
-Nothing but c and k_r is cached, and keys are never expanded: q_plain . (W_uk,h c) = (q_plain W_uk,h) . c,
-so attention runs over the latents as one shared key/value head of kv_rank + rot_dim numbers with
-W_uk folded into the queries, and W_uv is applied to the attention's output.  The cache is then what the
-attention kernels of the other mixers read: keys [c | k_r], values c, padded to a multiple of 16.
+Nothing but c and k_r is cached, and keys are never expanded: q_plain . (W_uk,h c) = (W_uk,h^T q_plain) . c,
+so attention runs over the latents as one shared key/value head of kv_rank + rot_dim numbers, and W_uv is
+applied to the attention's output.  W_uk is folded into the query up-projection once, when the weights are
+loaded: head h of the folded matrix is [W_uk,h^T W_uq,h(plain rows) ; W_uq,h(rotated rows) ; 0], so that one
+product gives every head's query against the cache's key rows [c | k_r | 0] and only the rotation is left to do.
+The cache is what the attention kernels of the other mixers read: keys [c | k_r], values c, padded to a multiple of 16.
 
 A layer built with ``has_kv`` False has no W_dkv: it reads another layer call's cache (same kv_rank,
 rot_dim and position encoding) with its own W_uk, W_uv and queries.
@@ -18,7 +20,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass
 
-from .base import CacheRequirement, Mixer, ParamSpec, Source, register_mixer
+from .base import CacheRequirement, Mixer, ParamSpec, register_mixer
 
 DEFAULT_NAMES = dict(dq="dq", dq_norm="dq.norm", uq="uq", dkv="dkv", dkv_norm="dkv.norm", uk="uk", uv="uv", g="g", o="o")
 
@@ -63,6 +65,7 @@ class LatentAttention(Mixer):
         self.names = dict(DEFAULT_NAMES, **(tensor_names or {}))
         if position.rotary_dim > self.rot_dim:
             raise ValueError(f"the position encoding turns {position.rotary_dim} dims; the rotated part has {self.rot_dim}")
+        self.w_uq = self.w_uk = self.w_q = None
         self.padded_dim = PagedLatent(self.kv_rank, self.rot_dim).padded_dim
         if self.padded_dim > self.MAX_PADDED_DIM:
             raise ValueError(f"kv_rank {kv_rank} + rot_dim {rot_dim} is beyond the {self.MAX_PADDED_DIM} numbers a token "
@@ -82,10 +85,7 @@ class LatentAttention(Mixer):
         specs = [ParamSpec.stacked("w_down", down),
                  ParamSpec.single("dq_norm", name("dq_norm"), (self.q_rank,), init="scale"),
                  ParamSpec.single("w_uq", name("uq"), (H * (self.dim + self.rot_dim), self.q_rank)),
-                 # W_uk is folded into the queries, head by head: kept transposed, [kv_rank, H dim]
-                 ParamSpec("w_uk_t", (self.kv_rank, H * self.dim),
-                           (Source(name("uk"), (self.kv_rank, H * self.dim), 0, stored_shape=(H * self.dim, self.kv_rank),
-                                   transform="transpose"),)),
+                 ParamSpec.single("w_uk", name("uk"), (H * self.dim, self.kv_rank)),
                  ParamSpec.single("w_uv", name("uv"), (H * self.vdim, self.kv_rank)),
                  ParamSpec.single("w_o", name("o"), (w, H * self.vdim))]
         if self.has_kv:
@@ -94,6 +94,20 @@ class LatentAttention(Mixer):
 
     def cache_requirement(self):
         return PagedLatent(self.kv_rank, self.rot_dim)
+
+    def prepare(self, device, dtype):
+        """Fold W_uk into W_uq (in 32-bit, rounded once to the weights' dtype); the two are not needed afterwards."""
+        import torch
+        if self.w_uq is None:
+            return
+        H, d, dr, r, P = self.num_heads, self.dim, self.rot_dim, self.kv_rank, self.padded_dim
+        uq = self.w_uq.float().view(H, d + dr, self.q_rank)
+        uk = self.w_uk.float().view(H, d, r)
+        folded = torch.zeros((H, P, self.q_rank), dtype=torch.float32, device=self.w_uq.device)
+        folded[:, :r] = torch.einsum("hdr,hdq->hrq", uk, uq[:, :d])
+        folded[:, r:r + dr] = uq[:, d:]
+        self.w_q = folded.view(H * P, self.q_rank).to(self.w_uq.dtype).contiguous()
+        self.w_uq = self.w_uk = None
 
     def forward(self, x, step, cache, add_to=None):
         import torch
@@ -107,14 +121,14 @@ class LatentAttention(Mixer):
         # one product for everything that reads x: query latent, key/value latent + rotated key part, gate
         sums = ops.linear(x, self.w_down, out_dtype=torch.float32)
         col = self.q_rank
-        if self.has_kv:
-            ops.latent_kv_store(sums, col, self.kv_rank, self.rot_dim, self.dkv_norm, self.eps, step.positions, inv_freq,
-                                cache.k, cache.v, group.slot_mapping)
+        if self.has_kv:      # the token's cache entry and, in the same kernel, its normed query latent
+            cq = ops.latent_kv_store(sums, col, self.kv_rank, self.rot_dim, self.dkv_norm, self.eps, step.positions, inv_freq,
+                                     cache.k, cache.v, group.slot_mapping, also_norm=(0, self.q_rank, self.dq_norm))
             col += self.kv_rank + self.rot_dim
-        cq = ops.rmsnorm_columns(sums, 0, self.q_rank, self.dq_norm, self.eps)
-        q = ops.linear(cq, self.w_uq)
-        q = ops.latent_query(q, self.w_uk_t, self.num_heads, self.dim, self.rot_dim, self.kv_rank, step.positions, inv_freq,
-                             self.padded_dim)
+        else:
+            cq = ops.rmsnorm_columns(sums, 0, self.q_rank, self.dq_norm, self.eps)
+        q = ops.latent_query_rotate_(ops.linear(cq, self.w_q), self.num_heads, self.kv_rank, self.padded_dim, step.positions,
+                                     inv_freq)
         o = ops.paged_attention(q, self.num_heads, 1, self.padded_dim, cache.k, cache.v, group, step, self.scale, None)
         heads = ops.latent_value_gate(o, self.w_uv, sums if self.gated else None, col, self.num_heads, self.vdim,
                                       self.kv_rank, self.padded_dim)

@@ -446,14 +446,19 @@ def test_latent_attention_kernels(hip, dtype):
         vc = torch.full((pages, 1, P, page), 7.0, dtype=dtype).cuda()
         kw, vw = kc.clone(), vc.clone()
         ref.ref_latent_kv_store(sums, 11, r, rot, nw, 1e-5, positions, inv_freq, kw, vw, slots)
-        ops.latent_kv_store(sums, 11, r, rot, nw, 1e-5, positions, inv_freq, kc, vc, slots)
+        qw = _rand((9,), dtype, g) + 1
+        cq = ops.latent_kv_store(sums, 11, r, rot, nw, 1e-5, positions, inv_freq, kc, vc, slots, also_norm=(1, 9, qw))
+        close(cq, ref.ref_rmsnorm_columns(sums, 1, 9, qw, 1e-5, dtype), TOL[dtype], "query latent normed beside")
         close(kc, kw, TOL[dtype], "keys")
         close(vc, vw, TOL[dtype], "values")
         assert torch.equal(kc[0], kw[0]), "the scratch page was not written"
-        q = _rand((T, H * (dim + rot)), dtype, g)
-        w_uk_t = _rand((r, H * dim), dtype, g, 0.3)
-        close(ops.latent_query(q, w_uk_t, H, dim, rot, r, positions, inv_freq, P),
-              ref.ref_latent_query(q, w_uk_t, H, dim, rot, r, positions, inv_freq, P, dtype), TOL[dtype], "query")
+        q = _rand((T, H * P), dtype, g)
+        want = ref.ref_latent_query_rotate(q.clone(), H, r, P, positions, inv_freq)
+        assert ops.latent_query_rotate_(q, H, r, P, positions, inv_freq) is q
+        close(q, want, TOL[dtype], "query rotation")
+        untouched = torch.ones(P, dtype=torch.bool)
+        untouched[r:r + 2 * n_freq] = False
+        assert torch.equal(q.view(T, H, P)[..., untouched], want.view(T, H, P)[..., untouched]), "only the turned pairs change"
         o = _rand((T, H * P), dtype, g)
         w_uv = _rand((H * vdim, r), dtype, g, 0.3)
         gate = _rand((T, 7 + H * vdim), torch.float32, g, 2.0)

@@ -66,13 +66,11 @@ def ref_latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions
     v_cache[page, 0, :kv_rank, off] = c.to(v_cache.dtype)
 
 
-def ref_latent_query(q, w_uk_t, H, dim, rot_dim, kv_rank, positions, inv_freq, padded, out_dtype):
-    T = q.shape[0]
-    qh = q.double().view(T, H, dim + rot_dim)
-    out = torch.zeros(T, H, padded, dtype=torch.float64, device=q.device)
-    out[..., :kv_rank] = torch.einsum("thd,rhd->thr", qh[..., :dim], w_uk_t.double().view(kv_rank, H, dim))
-    out[..., kv_rank:kv_rank + rot_dim] = ref_turn_pairs(qh[..., dim:], positions, inv_freq)
-    return out.view(T, H * padded).to(out_dtype)
+def ref_latent_query_rotate(q, H, kv_rank, padded, positions, inv_freq):
+    T, n = q.shape[0], 2 * inv_freq.shape[0]
+    heads = q.view(T, H, padded)
+    heads[..., kv_rank:kv_rank + n] = ref_turn_pairs(heads[..., kv_rank:kv_rank + n].double(), positions, inv_freq).to(q.dtype)
+    return q
 
 
 def ref_latent_value_gate(o, w_uv, gate, gate_col, H, vdim, kv_rank, padded, out_dtype):
@@ -280,12 +278,15 @@ class TorchBackend(KernelBackend):
         return (ref_act(gu[:, :intermediate], activation) * gu[:, intermediate:]).to(self.act_dtype)
 
     def latent_kv_store(self, sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache,
-                        slot_mapping):
+                        slot_mapping, also_norm=None):
         self._count("latent_kv_store")
         ref_latent_kv_store(sums, col, kv_rank, rot_dim, norm_weight, eps, positions, inv_freq, k_cache, v_cache, slot_mapping)
+        if also_norm is not None:
+            return ref_rmsnorm_columns(sums, also_norm[0], also_norm[1], also_norm[2], eps, self.act_dtype)
+        return None
 
-    def latent_query(self, q, w_uk_t, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim):
-        return ref_latent_query(q, w_uk_t, num_heads, dim, rot_dim, kv_rank, positions, inv_freq, padded_dim, self.act_dtype)
+    def latent_query_rotate_(self, q, num_heads, kv_rank, padded_dim, positions, inv_freq):
+        return ref_latent_query_rotate(q, num_heads, kv_rank, padded_dim, positions, inv_freq)
 
     def latent_value_gate(self, o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim):
         return ref_latent_value_gate(o, w_uv, gate, gate_col, num_heads, vdim, kv_rank, padded_dim, self.act_dtype)
