@@ -36,7 +36,8 @@ def build_zifelorn(cfg: ZifelornConfig) -> DecoderSpec:
         else:
             norm2 = RMSNorm(w, eps, f"{p}.norm2")
             if isinstance(f, DenseFFSpec):
-                ff = SwiGLU(w, f.ff, prefix=f"{p}.mlp", activation="gelu_tanh", tensor_names=("gate", "up", "down"))
+                ff = SwiGLU(w, f.ff, prefix=f"{p}.mlp", activation="gelu_tanh", tensor_names=("gate", "up", "down"),
+                            float32_output=True)
             elif isinstance(f, MoEFFSpec):
                 ff = RoutedExperts(w, f.expert_ff, f.experts, f.top, prefix=f"{p}.mlp", activation="relu2")
             else:

@@ -12,7 +12,7 @@ class SwiGLU(FeedForward):
     lazy_input = True
 
     def __init__(self, width: int, intermediate: int, prefix: str, activation: str = "silu",
-                 tensor_names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+                 tensor_names=("gate_proj.weight", "up_proj.weight", "down_proj.weight"), float32_output: bool = False):
         from ..kernels.api import ACTIVATIONS
         if activation not in ACTIVATIONS:
             raise ValueError(f"activation {activation!r}: one of {ACTIVATIONS}")
@@ -21,6 +21,7 @@ class SwiGLU(FeedForward):
         self.prefix = prefix
         self.activation = activation
         self.tensor_names = tuple(tensor_names)
+        self.float32_output = bool(float32_output)      # where the caller norms the output itself: hand it the 32-bit sums
         self.w_gate_up = None
         self.w_down = None
 
@@ -35,4 +36,7 @@ class SwiGLU(FeedForward):
             a = self.ops.linear_silu_mul(x, self.w_gate_up, self.intermediate)
         else:
             a = self.ops.linear_act_mul(x, self.w_gate_up, self.intermediate, self.activation)
+        if self.float32_output and add_to is None:
+            import torch
+            return self.ops.linear(a, self.w_down, out_dtype=torch.float32)
         return self.ops.linear(a, self.w_down, add_to=add_to)

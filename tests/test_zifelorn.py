@@ -275,13 +275,13 @@ def test_families_on_the_host(name, family, tmp_path):
     run_family(name, family, tmp_path, "cpu", "float32", F32_TOL)
 
 
-def test_a_far_key_and_the_first_token_are_seen(tmp_path):
-    """One head's query is made to point at the key of one far token (and, in a second run, of the very first):
-    the plain implementation then puts nearly all weight there, and so must the engine, through 13 pages and
-    across portions and single tokens."""
+def far_key_runs(device):
+    """One token is made to stand out (an embedding no other position has): far back, at the last slot of a page and the
+    first of the next, and at the very first position.  The engine must follow the plain implementation through 13
+    pages, a portion of 150 tokens and 50 single tokens; and the token must matter to the last position."""
     raw, cfg, weights = make("A")
     toks = [t if t != 210 else 0 for t in trace_util.random_prompts(raw["vocab"], [200], seed=9)["r0"]]
-    for needle in (37, 0):
+    for needle in (37, 15, 16, 0):
         tokens = list(toks)
         tokens[needle] = 210                                   # a token no other position holds
         assert tokens.count(210) == 1
@@ -292,14 +292,26 @@ def test_a_far_key_and_the_first_token_are_seen(tmp_path):
         steps += [{"step": 1 + i, "entries": [{"id": "x", "tokens": tokens[150 + i:151 + i], "want": [0]}], "end": []}
                   for i in range(50)]
         steps[-1]["end"] = ["x"]
-        runner = host_runner(cfg, w, pages=16, rows=2, tokens=160)
-        got = trace_util.run_on_runner(runner, steps)
+        if device == "cpu":
+            runner = host_runner(cfg, w, pages=16, rows=2, tokens=160)
+        else:
+            runner = ModelRunner(cfg, weights=w, dtype="float32", num_pages=16, max_rows=2, max_step_tokens=160, max_model_len=240)
+        got = {k: v.cpu() for k, v in trace_util.run_on_runner(runner, steps).items()}
         trace_util.compare(got, {"x": want}, F32_TOL, f"needle at {needle}")
         # and the needle matters: without it the last logits are different
         other = list(tokens)
         other[needle] = toks[needle]
         moved = float((plain.forward(raw, w, other)[-1] - want[-1]).abs().max()) / float(want.abs().max())
         assert moved > 1e-3, "the far token must matter to the last position for this test to mean anything"
+
+
+def test_a_far_key_and_the_first_token_are_seen():
+    far_key_runs("cpu")
+
+
+@pytest.mark.gpu
+def test_a_far_key_and_the_first_token_are_seen_gpu():
+    far_key_runs("cuda")
 
 
 def test_state_slots_and_pages_are_used_again(tmp_path):
@@ -472,7 +484,9 @@ def test_latent_attention_kernels(hip, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_recurrence_kernels(hip, dtype):
     ops, g = hip[dtype], torch.Generator().manual_seed(3)
-    for (C, B, K, lens, slots) in ((96, 3, 4, [1, 1, 9, 2, 300], [4, 1, 3, 5, 2]), (40, 5, 1, [5, 1], [1, 2]), (520, 1, 6, [3, 2, 40], [2, 3, 1])):
+    # rows of 32, 33, 64 and 65 tokens: the scan's chunks are 32 long, and a row of up to 32 runs in one pass
+    for (C, B, K, lens, slots) in ((96, 3, 4, [1, 1, 9, 2, 300], [4, 1, 3, 5, 2]), (40, 5, 1, [5, 1], [1, 2]), (520, 1, 6, [3, 2, 40], [2, 3, 1]),
+                                   (64, 2, 3, [32, 33, 64, 65, 1], [5, 4, 3, 2, 1]), (64, 2, 3, [32, 2], [1, 2])):
         step = FakeStep(lens, slots)
         T = step.num_tokens
         x = _rand((T, 2 * C + 3), torch.float32, g)
