@@ -57,7 +57,13 @@ CFG_B = dict(architecture="Zifelorn", vocab=150, width=48, embedding=dict(scale=
                      layer("latent_attention", B1, None),
                      layer("latent_attention", dict(B1, kv_from=1), moe(6, 4, 16)),
                      layer("rglru", dict(width=48, blocks=2, conv=6), dict(kind="dense", ff=64))])
-CONFIGS = {"A": (CFG_A, 3), "B": (CFG_B, 4)}
+# sizes the kernels' vector paths do not like: nothing a multiple of 8, an odd vocabulary
+C1 = att(3, 10, 6, 14, 22, 18, base=300.0)
+CFG_C = dict(architecture="Zifelorn", vocab=101, width=70, embedding=dict(scale=3.0), norm=dict(eps=1e-6), logit_scale=1.3,
+             layers=[layer("latent_attention", C1, moe(3, 2, 26)),
+                     layer("rglru", dict(width=30, blocks=3, conv=3), dict(kind="dense", ff=50)),
+                     layer("latent_attention", dict(C1, kv_from=0), dict(kind="dense", ff=34))])
+CONFIGS = {"A": (CFG_A, 3), "B": (CFG_B, 4), "C": (CFG_C, 6)}
 
 
 def make(name, dtype=torch.float32, sharp=True):
