@@ -55,7 +55,7 @@ class CacheStorage:
         idx = torch.tensor(list(pages), dtype=torch.long, device=self.device)
         for t in self.entries.values():
             if t.group == group:
-                for x in t.tensors.values():
+                for x in t.requirement.paged_tensors(t.tensors):
                     if x.is_floating_point():
                         x.index_fill_(0, idx, float("nan"))
 

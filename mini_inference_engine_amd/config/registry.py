@@ -98,7 +98,32 @@ def architecture_of(config: ModelConfig) -> Architecture:
     return _ARCHITECTURES[name]
 
 
-def load_model_config(path_or_dict) -> tuple[ModelConfig, Architecture]:
+def checkpoint_tensor_shapes(folder: str) -> dict:
+    """name -> shape of every tensor in the folder's safetensors files, from the files' headers alone (eight bytes
+    of length, little-endian, then that many bytes of JSON)."""
+    import glob
+    import json
+    import os
+    import struct
+    shapes = {}
+    for fn in sorted(glob.glob(os.path.join(folder, "*.safetensors"))):
+        with open(fn, "rb") as f:
+            (n,) = struct.unpack("<Q", f.read(8))
+            header = json.loads(f.read(n))
+        for name, entry in header.items():
+            if name != "__metadata__":
+                shapes[name] = tuple(entry["shape"])
+    return shapes
+
+
+def load_model_config(path_or_dict, tensor_shapes=None) -> tuple[ModelConfig, Architecture]:
+    """``tensor_shapes`` (name -> shape): for a configuration type that takes some size from the checkpoint's tensors
+    rather than from a key (``reads_tensor_shapes``); read from the folder's files where a folder is given."""
     d = path_or_dict if isinstance(path_or_dict, Mapping) else read_config_json(path_or_dict)
     arch = architecture_for(d)
+    if getattr(arch.config_type, "reads_tensor_shapes", False):
+        if tensor_shapes is None and not isinstance(path_or_dict, Mapping):
+            import os
+            tensor_shapes = checkpoint_tensor_shapes(path_or_dict if os.path.isdir(path_or_dict) else os.path.dirname(path_or_dict))
+        return arch.config_type.from_dict(d, tensor_shapes=tensor_shapes), arch
     return arch.config_type.from_dict(d), arch

@@ -169,6 +169,49 @@ class KernelBackend:
         w_down [E, width, ff]; the hidden activation is rounded once to the activation dtype -> [T, width] float32."""
         raise NotImplementedError
 
+    # ---- a short convolution on a mixer's input, attention from one product's sums, the delta rule
+    def residual_conv(self, h, taps, tail, step, out_dtype=None):
+        """h [T, C] float32, taps [C, K] float32: y[t] = h[t] + sum_j taps[:, j] * h[t - (K - 1) + j], per row of the
+        step; inputs before a row's first token come from ``tail`` [slots, max(1, K - 1), C] float32 (the last K - 1
+        inputs of the row's request, oldest first; zeros at its start), which afterwards holds the last K - 1 inputs
+        including this step's.  All float32 -> [T, C] in ``out_dtype`` (default: the activation dtype)."""
+        raise NotImplementedError
+
+    def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
+                   layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None):
+        """What lies between a q/k/v projection's float32 sums [T, *] and attention, in 32-bit: queries are columns
+        [q_col, q_col + Hq dim), keys [k_col, k_col + Hkv dim), values [v_col, v_col + Hkv vdim), or, with ``v_col``
+        None, the keys as projected (vdim = dim).  ``q_norm`` / ``k_norm`` (float32 [Hq dim] / [Hkv dim]): RMS norm over
+        the whole of a token's queries (keys) at once, times that weight, before anything else.  Then the first
+        2 * len(inv_freq) numbers of every query and key head turn by the angles position * inv_freq[i]: ``layout``
+        "interleaved" pairs (2i, 2i + 1), "half" pairs (i, i + len(inv_freq)).  ``q_head_scale`` (float32 [Hq]):
+        head h's turned query times that number.  Keys and values go to the token's slot of k_cache [pages, Hkv, page, P]
+        and v_cache [pages, Hkv, P, page], P = ``padded_dim`` >= dim, vdim, zeros beyond their own size.
+        -> q [T, Hq * P] in the activation dtype, zeros beyond dim."""
+        raise NotImplementedError
+
+    def head_gate_(self, o, gate, gate_col, num_heads, head_dim):
+        """o [T, H * head_dim] *= sigmoid(gate[t, gate_col + h]) for every number of head h, in place (gate float32
+        [T, *]).  Returns o."""
+        raise NotImplementedError
+
+    def delta_rule(self, sums, cols, num_heads, dim, w_decay, decay_bias, decay_scale, removal_bias, norm_weight, eps,
+                   state, step):
+        """The delta-rule recurrence from one product's float32 sums [T, *].  ``cols``: first column of r, k, v (H dim
+        each), of the output gate g and the removal gate a (H dim each) and of the decay's inner activations w
+        (w_decay.shape[1] of them).  Per token, head and key channel i, all in 32-bit:
+        decay = exp(-decay_scale * sigmoid(w_decay tanh(w) + decay_bias)), a = sigmoid(a + removal_bias),
+        u = k / sqrt(sum(k^2) + 1e-6) per head.  Per row and head, tokens in order, from the row's slot of ``state``
+        [slots, H, dim, dim] float32 (S[i, j]: key channel i, value channel j), left there afterwards:
+        S <- diag(decay) S - (a * u) (u^T S) + k v^T with both terms of the old S; o = S^T r.
+        -> rmsnorm(o over a head, eps) * norm_weight * sigmoid(g)  [T, H * dim] in the activation dtype."""
+        raise NotImplementedError
+
+    def normed_sum_add(self, stream, ys, weights, eps, scale):
+        """stream += scale * sum_i rmsnorm(ys[i], eps) * weights[i], row by row in float32 (each y [T, width] float32,
+        one or two of them).  Returns stream."""
+        raise NotImplementedError
+
     def rotary_kv_store(self, qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
                         k_cache, v_cache, slot_mapping):
         """Rotate the first ``rotary_dim`` dims of every q and k head of
@@ -191,11 +234,12 @@ class KernelBackend:
         return qkv
 
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
-                        window):
+                        window, sink=None):
         """For token t of row r at position p: softmax over keys max(0, p - window + 1)..p
         of row r (read through group.block_tables[r]) of (q . k) * scale, times v.
         q head i uses kv head i // (Hq / Hkv).  q is the first Hq * D columns of
-        qkv (row stride qkv.stride(0)).  Returns [T, Hq * D] in act_dtype."""
+        qkv (row stride qkv.stride(0)).  ``sink`` (a number): one more term exp(sink) in every softmax's
+        denominator, with no value.  Returns [T, Hq * D] in act_dtype."""
         raise NotImplementedError
 
     def sample(self, logits, temperatures, seeds, counters, out=None):

@@ -31,7 +31,7 @@ class Decoder:
         for e, call in enumerate(spec.schedule):
             if call.cache_of is not None:
                 continue
-            req = spec.layers[call.layer].mixer.cache_requirement()
+            req = spec.layers[call.layer].cache_requirement()
             if req is None:
                 continue
             if not isinstance(req, CacheRequirement):
@@ -47,7 +47,7 @@ class Decoder:
         self.bindings: list[CacheBinding] = []
         # whether a step may carry padding tokens (written to the scratch page): not if a mixer keeps state that
         # every token of a row changes
-        self.padding_safe = all(ce.requirement.paged for ce in self.cache_entries.values())
+        self.padding_safe = not any(ce.requirement.stateful for ce in self.cache_entries.values())
 
     # ------------------------------------------------------------ structure
     def parts(self):

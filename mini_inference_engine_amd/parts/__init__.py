@@ -1,13 +1,17 @@
 from .attention import Attention
-from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Block, CacheBinding, CacheRequirement, DecoderSpec,
+from .base import (BLOCKS, CombinedCache, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Block, CacheBinding, CacheRequirement, DecoderSpec,
                    FeedForward, FixedState, LayerCall, Mixer, Norm, PagedKV, ParamSpec, Part, PositionEncoding,
                    Source, WEIGHT_TRANSFORMS, register_block, register_feed_forward, register_mixer, register_norm,
                    register_position_encoding, register_weight_transform)
-from .block import BranchNormBlock, PreNormBlock
+from .block import BranchNormBlock, ParallelBlock, PreNormBlock
+from .delta_rule import DeltaRule
 from .embedding import Embedding, LMHead
+from .input_conv import ConvTail, ResidualConv
 from .latent_attention import LatentAttention, PagedLatent
 from .rglru import RGLRU, RecurrentState
 from .rmsnorm import RMSNorm
-from .rope import NoPosition, RotaryHalfSplit, RotaryInterleaved, rotary_tables
+from .rope import NoPosition, RotaryHalfAngles, RotaryHalfSplit, RotaryInterleaved, rotary_tables
 from .routed_experts import RoutedExperts
+from .side_by_side import SideBySide
+from .softmax_attention import SoftmaxAttention
 from .swiglu import SwiGLU

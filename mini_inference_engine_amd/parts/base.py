@@ -151,6 +151,16 @@ class CacheRequirement:
     paged = False
     window = None
 
+    @property
+    def stateful(self) -> bool:
+        """Whether the entry keeps state of fixed size in the request's state slot (every token of a row changes
+        it, so a step may carry no padding tokens, and a slot handed to a request is reset first)."""
+        return not self.paged
+
+    def paged_tensors(self, tensors: dict) -> list:
+        """Those of ``allocate``'s tensors whose first index is a page id."""
+        return list(tensors.values()) if self.paged else []
+
     def page_group_key(self):
         return self.window
 
@@ -199,6 +209,67 @@ class FixedState(CacheRequirement):
         tensors["state"][slot].zero_()
 
 
+class CombinedCache(CacheRequirement):
+    """What a layer call keeps when several of its parts keep something: named requirements side by side (a mixer
+    beside a convolution's last inputs; two mixers that read the same input).  At most one of them, however deep,
+    may be paged (a layer call has one block table); its window and page group are the combination's.  The tensors
+    are allocated under ``<name>.<tensor>``; ``CacheBinding.sub(name)`` gives a part the binding it would have
+    had alone."""
+
+    def __init__(self, members):
+        self.members = tuple((str(n), r) for n, r in members if r is not None)
+        paged = [r for _, r in self.members if r.paged]
+        if len(paged) > 1:
+            raise ValueError("a layer call can keep only one kind of data in pages")
+        self._paged = paged[0] if paged else None
+
+    def __eq__(self, other):
+        return isinstance(other, CombinedCache) and self.members == other.members
+
+    def __hash__(self):
+        return hash(self.members)
+
+    def __repr__(self):
+        return f"CombinedCache({dict(self.members)!r})"
+
+    @property
+    def paged(self):
+        return self._paged is not None
+
+    @property
+    def window(self):
+        return self._paged.window if self._paged is not None else None
+
+    @property
+    def stateful(self):
+        return any(r.stateful for _, r in self.members)
+
+    def page_group_key(self):
+        return self._paged.page_group_key() if self._paged is not None else None
+
+    def bytes_per_page(self, page_size, element_size):
+        return self._paged.bytes_per_page(page_size, element_size) if self._paged is not None else 0
+
+    @staticmethod
+    def _of(tensors: dict, name: str) -> dict:
+        return {k[len(name) + 1:]: t for k, t in tensors.items() if k.startswith(name + ".")}
+
+    def allocate(self, num_pages, page_size, num_slots, device, act_dtype):
+        out = {}
+        for name, r in self.members:
+            for k, t in r.allocate(num_pages, page_size, num_slots, device, act_dtype).items():
+                out[f"{name}.{k}"] = t
+        return out
+
+    def reset_slot(self, tensors, slot):
+        for name, r in self.members:
+            if r.stateful:
+                r.reset_slot(self._of(tensors, name), slot)
+
+    def paged_tensors(self, tensors):
+        return [t for name, r in self.members for t in r.paged_tensors(self._of(tensors, name))]
+
+
 @dataclass
 class CacheBinding:
     """What a mixer call gets: the tensors of the cache entry it reads/writes."""
@@ -209,6 +280,12 @@ class CacheBinding:
     read_only: bool = False           # entry belongs to another layer call
     page_size: int = 0
     tensors: Any = None               # everything the requirement allocated, by name
+
+    def sub(self, name: str) -> "CacheBinding":
+        """The binding of member ``name`` of a CombinedCache: its tensors under their own names."""
+        own = CombinedCache._of(self.tensors or {}, name)
+        return CacheBinding(group=self.group, k=own.get("k"), v=own.get("v"), state=own.get("state"),
+                            read_only=self.read_only, page_size=self.page_size, tensors=own)
 
 
 class Norm(Part):
@@ -253,6 +330,10 @@ class FeedForward(Part):
 class Block(Part):
     mixer: Mixer
     first_norm = None       # the norm a block applies to the stream first, if it wants the block before it to know
+
+    def cache_requirement(self):
+        """What a call of this block keeps between steps: its mixer's need, unless the block keeps more."""
+        return self.mixer.cache_requirement()
 
     def forward(self, h, residual, step, cache: CacheBinding, next_norm=None):
         raise NotImplementedError

@@ -8,7 +8,7 @@ be added: the next block's first norm (or the final norm) adds it
 from __future__ import annotations
 
 from ..kernels.api import Normed, Sink, StreamCopy
-from .base import Block, register_block
+from .base import Block, CombinedCache, register_block
 
 
 @register_block("pre_norm")
@@ -82,3 +82,55 @@ class BranchNormBlock(Block):
             y = self.feed_forward.forward(x, step)
             x = ops.branch_norm_add(y, residual, self.norm_feed_forward.weight, self.norm_feed_forward.eps)
         return StreamCopy(residual, x), residual
+
+
+@register_block("parallel")
+class ParallelBlock(Block):
+    """Mixer and feed-forward side by side, each behind a norm of its own of the same stream:
+    stream += mixer(c(norm_mixer(stream))) + feed_forward(norm_feed_forward(stream)).  ``input_conv`` (c, a
+    parts.ResidualConv, or None) is a short convolution on what the mixer reads; its last inputs are kept beside
+    the mixer's cache (CombinedCache members ``mixer`` and ``conv``).  ``feed_forward`` (and its norm) may be None.
+    Both norms are taken before either branch is added; the adds are 32-bit."""
+
+    def __init__(self, norm_mixer, mixer, norm_feed_forward=None, feed_forward=None, input_conv=None):
+        if (feed_forward is None) != (norm_feed_forward is None):
+            raise ValueError("a feed-forward and its norm come together or not at all")
+        self.norm_mixer, self.mixer = norm_mixer, mixer
+        self.norm_feed_forward, self.feed_forward = norm_feed_forward, feed_forward
+        self.input_conv = input_conv
+
+    def children(self):
+        return [p for p in (self.norm_mixer, self.input_conv, self.mixer, self.norm_feed_forward, self.feed_forward)
+                if p is not None]
+
+    def cache_requirement(self):
+        if self.input_conv is None:
+            return self.mixer.cache_requirement()
+        return CombinedCache([("mixer", self.mixer.cache_requirement()), ("conv", self.input_conv.cache_requirement())])
+
+    def forward(self, h, residual, step, cache, next_norm=None):
+        import torch
+        ops = self.ops
+        if isinstance(h, Normed):               # a block of another kind before this one: its last add may be pending
+            h = h.pending
+        elif isinstance(h, StreamCopy):
+            h = None
+        if h is not None:
+            residual.add_(h.float())
+        conv = self.input_conv
+        x = ops.add_rmsnorm(None, residual, self.norm_mixer.weight, self.norm_mixer.eps,
+                            out_dtype=torch.float32 if conv is not None else None)
+        if conv is not None:
+            x = conv.forward(x, step, cache.sub("conv"))
+        y = None
+        if self.feed_forward is not None:
+            y = ops.add_rmsnorm(None, residual, self.norm_feed_forward.weight, self.norm_feed_forward.eps)
+        sink = Sink(residual)
+        a = self.mixer.forward(x, step, cache.sub("mixer") if conv is not None else cache, add_to=sink)
+        if a is not None:
+            residual.add_(a.float())
+        if y is not None:
+            f = self.feed_forward.forward(y, step, add_to=sink)
+            if f is not None:
+                residual.add_(f.float())
+        return None, residual

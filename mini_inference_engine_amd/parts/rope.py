@@ -77,16 +77,28 @@ class RotaryInterleaved(PositionEncoding):
     compute the angle and its cosine and sine in 32-bit from the position and ``inv_freq`` [rotary_dim / 2]
     themselves, so there is no table and no longest position."""
 
-    def __init__(self, rotary_dim: int, theta: float):
+    layout = "interleaved"
+
+    def __init__(self, rotary_dim: int, theta: float, factor: float = 1.0):
+        """``factor``: linear scaling, every frequency divided by it."""
         self.rotary_dim = int(rotary_dim)
         self.theta = float(theta)
+        self.factor = float(factor)
         if self.rotary_dim % 2 or self.rotary_dim < 2:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and at least 2")
-        if not self.theta > 0:
-            raise ValueError("theta must be positive")
+        if not self.theta > 0 or not self.factor > 0:
+            raise ValueError("theta and the scaling factor must be positive")
         self.inv_freq = None
 
     def prepare(self, device, dtype):
         if self.inv_freq is None or self.inv_freq.device != torch.device(device):
             exponent = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64) / self.rotary_dim
-            self.inv_freq = (self.theta ** -exponent).to(torch.float32).to(device).contiguous()
+            self.inv_freq = (self.theta ** -exponent / self.factor).to(torch.float32).to(device).contiguous()
+
+
+@register_position_encoding("rotary_half_angles")
+class RotaryHalfAngles(RotaryInterleaved):
+    """The same angles on the other pairing: element i of the first ``rotary_dim`` dims turns with element
+    i + rotary_dim / 2.  Like RotaryInterleaved it keeps no table: the kernels that use it compute
+    position * inv_freq[i] and its cosine and sine in 32-bit themselves."""
+    layout = "half"

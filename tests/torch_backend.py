@@ -186,7 +186,7 @@ def ref_rotary_kv_store(qkv, positions, cos, sin, rotary_dim, Hq, Hkv, D, k_cach
 
 
 def ref_paged_attention(qkv, Hq, Hkv, D, k_cache, v_cache, block_tables, token_row, positions, scale, window,
-                        out_dtype):
+                        out_dtype, sink=None):
     """Token by token, keys gathered through the block table."""
     T = qkv.shape[0]
     P = k_cache.shape[2]
@@ -204,9 +204,107 @@ def ref_paged_attention(qkv, Hq, Hkv, D, k_cache, v_cache, block_tables, token_r
         v = v_cache[pages, :, :, keys % P].double()             # [n, Hkv, D]
         q = qkv[t, :Hq * D].double().view(Hkv, g, D)
         s = torch.einsum("hgd,nhd->hgn", q, k) * scale
-        pr = torch.softmax(s, dim=-1)
+        if sink is None:
+            pr = torch.softmax(s, dim=-1)
+        else:               # one more term in the denominator, with no value
+            top = s.max(-1, keepdim=True).values.clamp(min=sink)
+            e = torch.exp(s - top)
+            pr = e / (e.sum(-1, keepdim=True) + torch.exp(sink - top))
         out[t] = torch.einsum("hgn,nhd->hgd", pr, v).reshape(Hq * D).to(out_dtype)
     return out
+
+
+def ref_residual_conv(h, taps, tail, row_start, slots, out_dtype):
+    K = taps.shape[1]
+    out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
+    for r in range(len(slots)):
+        a, b, slot = int(row_start[r]), int(row_start[r + 1]), int(slots[r])
+        inp = torch.cat([tail[slot][:K - 1].double(), h[a:b].double()])
+        acc = h[a:b].double().clone()
+        for j in range(K):
+            acc += inp[j:j + b - a] * taps[:, j].double()
+        out[a:b] = acc.to(out_dtype)
+        if K > 1:
+            tail[slot][:K - 1] = inp[-(K - 1):].float()
+    return out
+
+
+def ref_turn(x, positions, inv_freq, layout):
+    """x [T, heads, d] float64: the first 2 * len(inv_freq) numbers of a head turn, adjacent pairs ("interleaved") or
+    element i with i + len(inv_freq) ("half"); the angle is a float32 product."""
+    if layout == "interleaved":
+        return ref_turn_pairs(x, positions, inv_freq)
+    n = inv_freq.shape[0]
+    angle = (positions.float()[:, None] * inv_freq.float()[None, :]).double()
+    c, s = angle.cos()[:, None, :], angle.sin()[:, None, :]
+    u, v = x[..., :n], x[..., n:2 * n]
+    out = x.clone()
+    out[..., :n] = u * c - v * s
+    out[..., n:2 * n] = v * c + u * s
+    return out
+
+
+def ref_qkv_finish(sums, q_col, k_col, v_col, Hq, Hkv, dim, vdim, P, positions, inv_freq, layout, k_cache, v_cache, slots,
+                   q_norm, k_norm, eps, q_head_scale, out_dtype):
+    T = sums.shape[0]
+    q = sums[:, q_col:q_col + Hq * dim].double()
+    k = sums[:, k_col:k_col + Hkv * dim].double()
+    v = k if v_col is None else sums[:, v_col:v_col + Hkv * vdim].double()
+    v = v.view(T, Hkv, -1)
+    if q_norm is not None:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm.double()
+    if k_norm is not None:
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm.double()
+    q, k = q.view(T, Hq, dim), k.view(T, Hkv, dim)
+    if inv_freq is not None:
+        q, k = ref_turn(q, positions, inv_freq, layout), ref_turn(k, positions, inv_freq, layout)
+    if q_head_scale is not None:
+        q = q * q_head_scale.double()[None, :, None]
+    page_size = k_cache.shape[2]
+    page, off = slots.long() // page_size, slots.long() % page_size
+    k_cache[page, :, off, :] = 0
+    k_cache[page, :, off, :dim] = k.to(k_cache.dtype)
+    v_cache[page, :, :, off] = 0
+    v_cache[page, :, :v.shape[-1], off] = v.to(v_cache.dtype)
+    out = torch.zeros(T, Hq, P, dtype=out_dtype, device=sums.device)
+    out[..., :dim] = q.to(out_dtype)
+    return out.view(T, Hq * P)
+
+
+def ref_head_gate(o, gate, gate_col, H, D):
+    T = o.shape[0]
+    g = torch.sigmoid(gate[:, gate_col:gate_col + H].double())
+    return (o.double().view(T, H, D) * g[:, :, None]).view(T, H * D).to(o.dtype)
+
+
+def ref_delta_rule(sums, cols, H, d, w_decay, decay_bias, decay_scale, removal_bias, norm_weight, eps, state, row_start, slots,
+                   out_dtype):
+    T, n = sums.shape[0], H * d
+    x = sums.double()
+    r, k, v, g, a = (x[:, cols[c]:cols[c] + n].view(T, H, d) for c in ("r", "k", "v", "g", "a"))
+    inner = torch.tanh(x[:, cols["w"]:cols["w"] + w_decay.shape[1]])
+    decay = torch.exp(-decay_scale * torch.sigmoid(inner @ w_decay.double().T + decay_bias.double())).view(T, H, d)
+    a = torch.sigmoid(a + removal_bias.double().view(H, d))
+    u = k * torch.rsqrt(k.pow(2).sum(-1, keepdim=True) + 1e-6)
+    out = torch.empty(T, H, d, dtype=torch.float64, device=sums.device)
+    for row in range(len(slots)):
+        S = state[int(slots[row])].double()
+        for t in range(int(row_start[row]), int(row_start[row + 1])):
+            seen = torch.einsum("hi,hij->hj", u[t], S)
+            S = decay[t][:, :, None] * S - (a[t] * u[t])[:, :, None] * seen[:, None, :] + k[t][:, :, None] * v[t][:, None, :]
+            out[t] = torch.einsum("hij,hi->hj", S, r[t])
+        state[int(slots[row])] = S.float()
+    out = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps)
+    return (out.view(T, n) * norm_weight.double() * torch.sigmoid(g.reshape(T, n))).to(out_dtype)
+
+
+def ref_normed_sum_add(stream, ys, weights, eps, scale):
+    total = torch.zeros_like(stream, dtype=torch.float64)
+    for y, w in zip(ys, weights):
+        yd = y.double()
+        total += yd * torch.rsqrt(yd.pow(2).mean(-1, keepdim=True) + eps) * w.double()
+    stream.add_((scale * total).float())
+    return stream
 
 
 def _fmix32(x):
@@ -340,10 +438,34 @@ class TorchBackend(KernelBackend):
                             k_cache, v_cache, slot_mapping)
 
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
-                        window):
+                        window, sink=None):
         self._count("paged_attention")
         return ref_paged_attention(qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group.block_tables,
-                                   step.token_row, step.positions, scale, window, self.act_dtype)
+                                   step.token_row, step.positions, scale, window, self.act_dtype, sink=sink)
+
+    def residual_conv(self, h, taps, tail, step, out_dtype=None):
+        self._count("residual_conv")
+        return ref_residual_conv(h, taps, tail, step.host["row_start"], step.host["state_slots"], out_dtype or self.act_dtype)
+
+    def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
+                   layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None):
+        self._count("qkv_finish")
+        return ref_qkv_finish(sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
+                              layout, k_cache, v_cache, slot_mapping, q_norm, k_norm, eps, q_head_scale, self.act_dtype)
+
+    def head_gate_(self, o, gate, gate_col, num_heads, head_dim):
+        o.copy_(ref_head_gate(o, gate, gate_col, num_heads, head_dim))
+        return o
+
+    def delta_rule(self, sums, cols, num_heads, dim, w_decay, decay_bias, decay_scale, removal_bias, norm_weight, eps,
+                   state, step):
+        self._count("delta_rule")
+        return ref_delta_rule(sums, cols, num_heads, dim, w_decay, decay_bias, decay_scale, removal_bias, norm_weight, eps,
+                              state, step.host["row_start"], step.host["state_slots"], self.act_dtype)
+
+    def normed_sum_add(self, stream, ys, weights, eps, scale):
+        self._count("normed_sum_add")
+        return ref_normed_sum_add(stream, ys, weights, eps, scale)
 
     def sample(self, logits, temperatures, seeds, counters, out=None):
         self._count("sample")
