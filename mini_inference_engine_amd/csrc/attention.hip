@@ -8,7 +8,8 @@
 // (one per lane: q . k in increasing d), the softmax is kept online in 32-bit, and the 64
 // probabilities then weight the value rows with the lanes spread over D.  The order of every
 // sum depends only on (lo, p): the result for a token is bit-identical whatever else the
-// step holds and however the request was cut into steps.
+// step holds and however the request was cut into steps.  With a sink, one more term exp(sink)
+// joins the softmax's denominator at the end and has no value.
 //
 // This is the reference kernel of the engine: the float32 path runs on it, and the
 // bfloat16 path uses it wherever a faster kernel does not take the shape.
@@ -40,7 +41,7 @@ __global__ void __launch_bounds__(64)
 paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restrict__ k_cache,
                        const T* __restrict__ v_cache, T* __restrict__ out, const int* __restrict__ block_tables,
                        int max_blocks, const int* __restrict__ token_row, const int* __restrict__ positions, int Hq,
-                       int Hkv, int D, int page, float scale, int window) {
+                       int Hkv, int D, int page, float scale, int window, int has_sink, float sink) {
   __shared__ float qs[NR * 64];
   __shared__ float ps[64];
   __shared__ long long base[64];     // per key of the chunk: offset of its value column
@@ -98,6 +99,13 @@ paged_attention_kernel(const T* __restrict__ q, long q_stride, const T* __restri
     __syncthreads();
     m = m_new;
   }
+  if (has_sink) {                     // one more term exp(sink) in the denominator, with no value
+    const float m_new = fmaxf(m, sink);
+    const float alpha = expf(m - m_new);
+    l = l * alpha + expf(sink - m_new);
+#pragma unroll
+    for (int i = 0; i < NR; ++i) acc[i] *= alpha;
+  }
   const float inv = 1.0f / l;
   T* op = out + ((size_t)t * Hq + h) * D;
 #pragma unroll
@@ -112,7 +120,7 @@ MIE_EXPORT const char* attention_last_error() { return g_mie_error; }
 MIE_EXPORT int mie_paged_attention(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
                                    int dtype, const int* block_tables, int max_blocks, const int* token_row,
                                    const int* positions, int tokens, int Hq, int Hkv, int D, int page, float scale,
-                                   int window, hipStream_t stream) {
+                                   int window, int has_sink, float sink, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (D % 16 || D < 16 || D > ATT_MAX_D) MIE_FAIL("paged_attention: head_dim %d (multiples of 16 up to %d)", D, ATT_MAX_D);
   if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("paged_attention: %d query heads on %d kv heads", Hq, Hkv);
@@ -123,7 +131,7 @@ MIE_EXPORT int mie_paged_attention(const void* q, long q_stride, const void* k_c
 #define PA_LAUNCH(T_, NR_)                                                                                               \
   hipLaunchKernelGGL((paged_attention_kernel<T_, NR_>), grid, block, 0, stream, (const T_*)q, q_stride, (const T_*)k_cache, \
                      (const T_*)v_cache, (T_*)out, block_tables, max_blocks, token_row, positions, Hq, Hkv, D, page, scale,  \
-                     window)
+                     window, has_sink, sink)
   if (dtype == MIE_F32 && D <= 256) PA_LAUNCH(float, 4);
   else if (dtype == MIE_F32) PA_LAUNCH(float, 16);
   else if (dtype == MIE_BF16 && D <= 256) PA_LAUNCH(bf16, 4);

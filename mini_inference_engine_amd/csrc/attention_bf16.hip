@@ -45,7 +45,8 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache
                         bf16* __restrict__ out, float* __restrict__ o_part,
                         float* __restrict__ lse_part, const int* __restrict__ block_tables, int max_blocks,
                         const int* __restrict__ positions, int Hq, int Hkv, int head_tiles, int page,
-                        float scale_log2, int window, int partition, int num_splits, ProjectionSums proj) {
+                        float scale_log2, int window, int partition, int num_splits, ProjectionSums proj,
+                        float sink_log2) {
   __shared__ float s_m[NW][16], s_l[NW][16], s_M[16], s_L[16];
   __shared__ float s_o[NW][16][D + 1];
   __shared__ __align__(16) bf16 s_q[FROM_SUMS ? 16 : 1][D];
@@ -305,11 +306,12 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < NW; ++w) sum += s_o[w][hc][d];
-    const float val = sum / s_L[hc];
     const size_t hh = (size_t)b * Hq + kvh * G + gg;
     if (num_splits == 1) {
-      out[hh * D + d] = __float2bfloat16(val);
+      // a sink (sink_log2 > -inf) is one more term in the denominator; with splits the merge kernel adds it
+      out[hh * D + d] = __float2bfloat16(sum / (s_L[hc] + exp2f(sink_log2 - s_M[hc])));
     } else {
+      const float val = sum / s_L[hc];
       o_part[(hh * num_splits + s) * D + d] = val;
       if (d == 0) lse_part[hh * num_splits + s] = s_M[hc] + log2f(s_L[hc]);
     }
@@ -323,7 +325,7 @@ decode_attention_kernel(const bf16* __restrict__ q, long q_stride, bf16* k_cache
 // cross the per-XCD L2s, and the device-scope fences that takes cost far more than this launch.)
 __global__ void __launch_bounds__(64)
 merge_splits_kernel(const float* __restrict__ o_part, const float* __restrict__ lse_part, bf16* __restrict__ out,
-                    int num_splits) {
+                    int num_splits, float sink_log2) {
   constexpr int DL = (D + 63) / 64;
   const size_t hh = blockIdx.x;
   const int lane = threadIdx.x;
@@ -369,7 +371,7 @@ merge_splits_kernel(const float* __restrict__ o_part, const float* __restrict__ 
       }
     }
   }
-  const float inv = 1.0f / W;
+  const float inv = 1.0f / (W + exp2f(sink_log2 - M));      // the sink's term, if there is one (else exp2(-inf) = 0)
 #pragma unroll
   for (int i = 0; i < DL; ++i) {
     const int d = lane + 64 * i;
@@ -384,10 +386,11 @@ MIE_EXPORT int mie_decode_block_keys() { return BLOCK_KEYS * NW_SPLIT; }
 // q: token b is row b (single-token rows lead the flattened batch).  partition: keys per split, a
 // multiple of mie_decode_block_keys().  o_part [rows, Hq, splits, D] and lse_part [rows, Hq, splits]
 // float are needed when num_splits > 1.
-MIE_EXPORT int mie_decode_attention(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
-                                    float* o_part, float* lse_part, const int* block_tables, int max_blocks,
-                                    const int* positions, int rows, int Hq, int Hkv, int head_dim, int page,
-                                    float scale, int window, int partition, int num_splits, hipStream_t stream) {
+static int decode_attention_launch(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                   float* o_part, float* lse_part, const int* block_tables, int max_blocks,
+                                   const int* positions, int rows, int Hq, int Hkv, int head_dim, int page,
+                                   float scale, int window, int partition, int num_splits, float sink_log2,
+                                   hipStream_t stream) {
   if (rows <= 0) return 0;
   if (head_dim != D) MIE_FAIL("decode_attention: built for head_dim %d, called with %d", D, head_dim);
   if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("decode_attention: %d query heads on %d kv heads", Hq, Hkv);
@@ -406,17 +409,37 @@ MIE_EXPORT int mie_decode_attention(const void* q, long q_stride, const void* k_
   if (num_splits == 1 && NW_WHOLE != NW_SPLIT && (long)rows * Hkv * head_tiles < NW_WHOLE_BELOW)
     hipLaunchKernelGGL((decode_attention_kernel<NW_WHOLE, false>), grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)q, q_stride,
                        kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
-                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{});
+                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{}, sink_log2);
   else
     hipLaunchKernelGGL((decode_attention_kernel<NW_SPLIT, false>), grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)q, q_stride,
                        kc, vc, (bf16*)out, o_part, lse_part, block_tables, max_blocks, positions, Hq, Hkv, head_tiles, page,
-                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{});
+                       scale * 1.4426950408889634f, window, partition, num_splits, ProjectionSums{}, sink_log2);
   MIE_CHECK_LAUNCH("decode_attention");
   if (num_splits > 1) {
-    hipLaunchKernelGGL(merge_splits_kernel, dim3(rows * Hq), dim3(64), 0, stream, o_part, lse_part, (bf16*)out, num_splits);
+    hipLaunchKernelGGL(merge_splits_kernel, dim3(rows * Hq), dim3(64), 0, stream, o_part, lse_part, (bf16*)out, num_splits,
+                       sink_log2);
     MIE_CHECK_LAUNCH("merge_splits");
   }
   return 0;
+}
+
+MIE_EXPORT int mie_decode_attention(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                    float* o_part, float* lse_part, const int* block_tables, int max_blocks,
+                                    const int* positions, int rows, int Hq, int Hkv, int head_dim, int page,
+                                    float scale, int window, int partition, int num_splits, hipStream_t stream) {
+  return decode_attention_launch(q, q_stride, k_cache, v_cache, out, o_part, lse_part, block_tables, max_blocks, positions,
+                                 rows, Hq, Hkv, head_dim, page, scale, window, partition, num_splits, -INFINITY, stream);
+}
+
+// The same with a sink: one more term exp(sink) in every softmax's denominator that has no value.
+MIE_EXPORT int mie_decode_attention_sink(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                         float* o_part, float* lse_part, const int* block_tables, int max_blocks,
+                                         const int* positions, int rows, int Hq, int Hkv, int head_dim, int page,
+                                         float scale, int window, int partition, int num_splits, float sink,
+                                         hipStream_t stream) {
+  return decode_attention_launch(q, q_stride, k_cache, v_cache, out, o_part, lse_part, block_tables, max_blocks, positions,
+                                 rows, Hq, Hkv, head_dim, page, scale, window, partition, num_splits,
+                                 sink * 1.4426950408889634f, stream);
 }
 
 
@@ -445,11 +468,11 @@ MIE_EXPORT int mie_decode_attention_from_sums(const float* part, int splits, lon
   if ((long)rows * Hkv < NW_WHOLE_BELOW)
     hipLaunchKernelGGL((decode_attention_kernel<NW_WHOLE, true>), grid, dim3(NW_WHOLE * 64), 0, stream, (const bf16*)nullptr, 0L,
                        (bf16*)k_cache, (bf16*)v_cache, (bf16*)out, (float*)nullptr, (float*)nullptr, block_tables, max_blocks,
-                       positions, Hq, Hkv, 1, page, scale * 1.4426950408889634f, window, partition, 1, proj);
+                       positions, Hq, Hkv, 1, page, scale * 1.4426950408889634f, window, partition, 1, proj, -INFINITY);
   else
     hipLaunchKernelGGL((decode_attention_kernel<NW_SPLIT, true>), grid, dim3(NW_SPLIT * 64), 0, stream, (const bf16*)nullptr, 0L,
                        (bf16*)k_cache, (bf16*)v_cache, (bf16*)out, (float*)nullptr, (float*)nullptr, block_tables, max_blocks,
-                       positions, Hq, Hkv, 1, page, scale * 1.4426950408889634f, window, partition, 1, proj);
+                       positions, Hq, Hkv, 1, page, scale * 1.4426950408889634f, window, partition, 1, proj, -INFINITY);
   MIE_CHECK_LAUNCH("decode_attention_from_sums");
   return 0;
 }

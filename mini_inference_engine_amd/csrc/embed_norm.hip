@@ -338,6 +338,36 @@ MIE_EXPORT int mie_rmsnorm_columns(const float* x, long ldx, const void* weight,
   return 0;
 }
 
+// ---- stream[row] += scale * (a * rstd(a) * wa + b * rstd(b) * wb): two branch outputs, each normed over the row, joined
+// and added in one pass (b null: one).  One workgroup a row, float32 throughout.
+__global__ void __launch_bounds__(NORM_THREADS)
+normed_sum_add_kernel(float* __restrict__ stream, const float* __restrict__ a, const float* __restrict__ wa,
+                      const float* __restrict__ b, const float* __restrict__ wb, int width, float eps, float scale) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * width;
+  float sa = 0.f, sb = 0.f;
+  for (int i = threadIdx.x; i < width; i += NORM_THREADS) {
+    sa = fmaf(a[base + i], a[base + i], sa);
+    if (b) sb = fmaf(b[base + i], b[base + i], sb);
+  }
+  const float ra = 1.0f / sqrtf(block_sum(sa, scratch) / (float)width + eps);
+  const float rb = b ? 1.0f / sqrtf(block_sum(sb, scratch) / (float)width + eps) : 0.f;
+  for (int i = threadIdx.x; i < width; i += NORM_THREADS) {
+    float v = a[base + i] * ra * wa[i];
+    if (b) v += b[base + i] * rb * wb[i];
+    stream[base + i] += scale * v;
+  }
+}
+
+MIE_EXPORT int mie_normed_sum_add(float* stream, const float* a, const float* wa, const float* b, const float* wb, int rows,
+                                  int width, float eps, float scale, hipStream_t s) {
+  if (rows <= 0) return 0;
+  if (width <= 0 || !stream || !a || !wa || (b && !wb)) MIE_FAIL("normed_sum_add: width %d or a missing operand", width);
+  hipLaunchKernelGGL(normed_sum_add_kernel, dim3(rows), dim3(NORM_THREADS), 0, s, stream, a, wa, b, wb, width, eps, scale);
+  MIE_CHECK_LAUNCH("normed_sum_add");
+  return 0;
+}
+
 // ---- t *= factor
 __global__ void scale_kernel(float* __restrict__ t, size_t n, float factor) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) t[i] *= factor;

@@ -74,7 +74,7 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
                          const bf16* __restrict__ v_cache, bf16* __restrict__ out,
                          const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ row_start,
                          const int* __restrict__ row_position, int first_row, int Hq, int Hkv, int waves_h,
-                         int page, float scale_log2, int window) {
+                         int page, float scale_log2, int window, float sink_log2) {
   extern __shared__ __align__(16) unsigned char pf_lds[];
   constexpr int PF_THREADS = PF_WAVES * 64;
   constexpr int SUB_WAVES = PF_WAVES / KS;                   // waves of one half
@@ -409,6 +409,7 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
         const float a0 = m == -INFINITY ? 0.f : fast_exp2(m - mj);
         const float a1 = m1 == -INFINITY ? 0.f : fast_exp2(m1 - mj);
         l = l * a0 + l1 * a1;
+        m = mj;
 #pragma unroll
         for (int dt = 0; dt < DT32; ++dt)
 #pragma unroll
@@ -418,7 +419,8 @@ prefill_attention_kernel(const bf16* __restrict__ q, long q_stride, const bf16* 
 
     const float total = pair_sum(l);
     if (q_ok && wk == 0) {
-      const float inv = 1.0f / total;
+      // a sink (sink_log2 > -inf) is one more term in the denominator; m is finite: a query sees its own key
+      const float inv = 1.0f / (total + fast_exp2(sink_log2 - m));
       bf16* op = out + ((size_t)qtok * Hq + head) * D + 4 * g;
 #pragma unroll
       for (int dt = 0; dt < DT32; ++dt)
@@ -440,10 +442,11 @@ MIE_EXPORT const char* prefill_attention_bf16_last_error() { return g_mie_error;
 
 // Rows first_row .. first_row + rows - 1 of the step (those of more than one token).  q and out are
 // indexed by flat token; row_start [all rows + 1], row_position [all rows] as the step gives them.
-MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
-                                     const int* block_tables, int max_blocks, const int* row_start,
-                                     const int* row_position, int first_row, int rows, int max_row_tokens, int Hq,
-                                     int Hkv, int head_dim, int page, float scale, int window, hipStream_t stream) {
+static int prefill_attention_launch(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                    const int* block_tables, int max_blocks, const int* row_start,
+                                    const int* row_position, int first_row, int rows, int max_row_tokens, int Hq,
+                                    int Hkv, int head_dim, int page, float scale, int window, float sink_log2,
+                                    hipStream_t stream) {
   if (rows <= 0 || max_row_tokens <= 0) return 0;
   if (head_dim != D) MIE_FAIL("prefill_attention: built for head_dim %d, called with %d", D, head_dim);
   if (Hkv <= 0 || Hq % Hkv) MIE_FAIL("prefill_attention: %d query heads on %d kv heads", Hq, Hkv);
@@ -497,7 +500,7 @@ MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k
     }
     hipLaunchKernelGGL(kernel, grid, dim3(waves * 64), lds_bytes, stream, (const bf16*)q, q_stride, (const bf16*)k_cache,
                        (const bf16*)v_cache, (bf16*)out, block_tables, max_blocks, row_start, row_position, first_row, Hq, Hkv,
-                       waves_h, page, scale_log2, window);
+                       waves_h, page, scale_log2, window, sink_log2);
     return 0;
   };
   int rc = 0;
@@ -509,4 +512,23 @@ MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k
   if (rc) return rc;
   MIE_CHECK_LAUNCH("prefill_attention");
   return 0;
+}
+
+MIE_EXPORT int mie_prefill_attention(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                     const int* block_tables, int max_blocks, const int* row_start,
+                                     const int* row_position, int first_row, int rows, int max_row_tokens, int Hq,
+                                     int Hkv, int head_dim, int page, float scale, int window, hipStream_t stream) {
+  return prefill_attention_launch(q, q_stride, k_cache, v_cache, out, block_tables, max_blocks, row_start, row_position,
+                                  first_row, rows, max_row_tokens, Hq, Hkv, head_dim, page, scale, window, -INFINITY, stream);
+}
+
+// The same with a sink: one more term exp(sink) in every softmax's denominator that has no value.
+MIE_EXPORT int mie_prefill_attention_sink(const void* q, long q_stride, const void* k_cache, const void* v_cache, void* out,
+                                          const int* block_tables, int max_blocks, const int* row_start,
+                                          const int* row_position, int first_row, int rows, int max_row_tokens, int Hq,
+                                          int Hkv, int head_dim, int page, float scale, int window, float sink,
+                                          hipStream_t stream) {
+  return prefill_attention_launch(q, q_stride, k_cache, v_cache, out, block_tables, max_blocks, row_start, row_position,
+                                  first_row, rows, max_row_tokens, Hq, Hkv, head_dim, page, scale, window,
+                                  sink * 1.4426950408889634f, stream);
 }

@@ -29,6 +29,41 @@ causal_conv_kernel(const float* __restrict__ x, long ldx, const float* __restric
   }
 }
 
+// residual_conv: y[t, c] = h[t, c] + sum_k taps[c, k] h[t - (K - 1 - k), c], no bias; inputs before the row's first
+// token come from tail[slot], which is only read here.  conv_tail_update, launched after it: the row's last K - 1
+// inputs (old tail, then this step's), oldest first, into tail[slot]; a thread a (row, channel), reads ahead of writes.
+template <typename TO>
+__global__ void __launch_bounds__(256)
+residual_conv_kernel(const float* __restrict__ h, const float* __restrict__ taps, const float* __restrict__ tail,
+                     const int* __restrict__ token_row, const int* __restrict__ row_start, const int* __restrict__ slots,
+                     TO* __restrict__ y, int C, int K) {
+  const int t = blockIdx.x;
+  const int r = token_row[t], j = t - row_start[r];
+  const float* tl = tail + (size_t)slots[r] * (K > 1 ? K - 1 : 1) * C;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
+    float acc = h[(size_t)t * C + c];
+    for (int k = 0; k < K; ++k) {
+      const int back = K - 1 - k;
+      const float v = back <= j ? h[(size_t)(t - back) * C + c] : tl[(size_t)(K - 1 + j - back) * C + c];
+      acc = fmaf(taps[(size_t)c * K + k], v, acc);
+    }
+    y[(size_t)t * C + c] = from_float<TO>(acc);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+conv_tail_update_kernel(const float* __restrict__ h, float* __restrict__ tail, const int* __restrict__ row_start,
+                        const int* __restrict__ slots, int C, int K) {
+  const int r = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= C) return;
+  const int a0 = row_start[r], n = row_start[r + 1] - a0, keep = K - 1;
+  float* tl = tail + (size_t)slots[r] * keep * C;
+  for (int i = 0; i < keep; ++i) {
+    const int src = n + i;                     // place in the joined sequence of keep + n inputs
+    tl[(size_t)i * C + c] = src < keep ? tl[(size_t)src * C + c] : h[(size_t)(a0 + src - keep) * C + c];
+  }
+}
+
 template <typename TO>
 __global__ void __launch_bounds__(256)
 rglru_scan_kernel(const float* __restrict__ u, const float* __restrict__ gates, const float* __restrict__ lam,
@@ -194,5 +229,26 @@ MIE_EXPORT int mie_rglru_scan(const float* u, const float* gates, const float* l
   else
     MIE_FAIL("rglru_scan: output dtype code %d", out_dtype);
   MIE_CHECK_LAUNCH("rglru_scan");
+  return 0;
+}
+
+// h [tokens, C] float32 contiguous; y [tokens, C] of y_dtype; tail [slots, max(1, K - 1), C] float32, read, then moved on.
+MIE_EXPORT int mie_residual_conv(const float* h, const float* taps, float* tail, const int* token_row, const int* row_start,
+                                 const int* slots, void* y, int y_dtype, int tokens, int rows, int C, int K, hipStream_t s) {
+  if (tokens <= 0 || rows <= 0) return 0;
+  if (C <= 0 || K < 1 || K > 64) MIE_FAIL("residual_conv: %d channels, %d taps (1 to 64)", C, K);
+  const int by = (C + 255) / 256 < 64 ? (C + 255) / 256 : 64;
+  if (y_dtype == MIE_F32)
+    hipLaunchKernelGGL(residual_conv_kernel<float>, dim3(tokens, by), dim3(256), 0, s, h, taps, tail, token_row, row_start,
+                       slots, (float*)y, C, K);
+  else if (y_dtype == MIE_BF16)
+    hipLaunchKernelGGL(residual_conv_kernel<bf16>, dim3(tokens, by), dim3(256), 0, s, h, taps, tail, token_row, row_start,
+                       slots, (bf16*)y, C, K);
+  else MIE_FAIL("residual_conv: out dtype code %d", y_dtype);
+  MIE_CHECK_LAUNCH("residual_conv");
+  if (K > 1) {
+    hipLaunchKernelGGL(conv_tail_update_kernel, dim3(rows, (C + 255) / 256), dim3(256), 0, s, h, tail, row_start, slots, C, K);
+    MIE_CHECK_LAUNCH("residual_conv (tail)");
+  }
   return 0;
 }

@@ -678,6 +678,126 @@ class HipBackend(KernelBackend):
         library.check(lib, lib.mie_moe_combine(_ptr(y), _ptr(place), _ptr(shares), _ptr(out), T, W, top, self._stream()))
         return out
 
+    # ---- a short convolution on a mixer's input, attention from one product's sums, the delta rule
+    def residual_conv(self, h, taps, tail, step, out_dtype=None):
+        self._on_device(h, taps, tail)
+        out_dtype = out_dtype or self.act_dtype
+        if h.dtype != torch.float32 or h.dim() != 2 or not h.is_contiguous():
+            raise ValueError("residual_conv: h must be contiguous float32 [T, channels]")
+        T, C = h.shape
+        if taps.dim() != 2 or taps.shape[0] != C:
+            raise ValueError(f"residual_conv: taps {tuple(taps.shape)} for {C} channels")
+        K = taps.shape[1]
+        self._f32_vector(taps, C * K, "residual_conv: taps")
+        if tail.dtype != torch.float32 or tuple(tail.shape[1:]) != (max(1, K - 1), C) or not tail.is_contiguous():
+            raise ValueError(f"residual_conv: tail {tuple(tail.shape)} for {K} taps of {C} channels")
+        self._check_rows("residual_conv", step, T)
+        if int(step.host["state_slots"].max()) >= tail.shape[0]:
+            raise ValueError("residual_conv: a state slot beyond the tail's slots")
+        y = torch.empty((T, C), dtype=out_dtype, device=h.device)
+        lib = self.lib("recurrence")
+        library.check(lib, lib.mie_residual_conv(_ptr(h), _ptr(taps), _ptr(tail), _ptr(step.token_row), _ptr(step.row_start),
+                                                 _ptr(step.state_slots), _ptr(y), _code(out_dtype), T, step.num_rows, C, K,
+                                                 self._stream()))
+        return y
+
+    LAYOUTS = {"interleaved": 0, "half": 1}
+
+    def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
+                   layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None):
+        self._on_device(sums, positions, inv_freq, k_cache, v_cache, slot_mapping, q_norm, k_norm, q_head_scale)
+        Hq, Hkv, P, T = num_q_heads, num_kv_heads, padded_dim, sums.shape[0]
+        if layout not in self.LAYOUTS:
+            raise ValueError(f"qkv_finish: layout {layout!r} (interleaved or half)")
+        self._f32_columns(sums, q_col, Hq * dim, "qkv_finish: queries")
+        self._f32_columns(sums, k_col, Hkv * dim, "qkv_finish: keys")
+        if v_col is not None:
+            self._f32_columns(sums, v_col, Hkv * vdim, "qkv_finish: values")
+        elif vdim != dim:
+            raise ValueError("qkv_finish: values that are the keys have the keys' size")
+        pages, hk, page, d = k_cache.shape
+        if (hk, d) != (Hkv, P) or tuple(v_cache.shape) != (pages, Hkv, P, page) or P < max(dim, vdim):
+            raise ValueError(f"qkv_finish: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} for {Hkv} kv heads of {P}")
+        if k_cache.dtype != self.act_dtype or v_cache.dtype != self.act_dtype or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+            raise ValueError("qkv_finish: caches must be contiguous and of the activation dtype")
+        nf = 0 if inv_freq is None else inv_freq.numel()
+        if nf:
+            self._f32_vector(inv_freq, nf, "qkv_finish: inv_freq")
+        if 2 * nf > dim:
+            raise ValueError(f"qkv_finish: {nf} turned pairs in heads of {dim}")
+        for name, t, n in (("q_norm", q_norm, Hq * dim), ("k_norm", k_norm, Hkv * dim), ("q_head_scale", q_head_scale, Hq)):
+            if t is not None:
+                self._f32_vector(t, n, f"qkv_finish: {name}")
+        for name, t in (("positions", positions), ("slot_mapping", slot_mapping)):
+            if t.dtype != torch.int32 or t.shape[0] != T or not t.is_contiguous():
+                raise ValueError(f"qkv_finish: {name} must be contiguous int32 [{T}]")
+        # rows 64 bytes apart from a multiple of their length, as the attention kernels like their q rows
+        q = torch.empty((T, Hq * P), dtype=self.act_dtype, device=sums.device)
+        lib = self.lib("attention_prep")
+        library.check(lib, lib.mie_qkv_finish(
+            _ptr(sums), sums.stride(0), q_col, k_col, -1 if v_col is None else v_col, _ptr(q_norm), _ptr(k_norm), float(eps),
+            _ptr(inv_freq), nf, self.LAYOUTS[layout], _ptr(q_head_scale), _ptr(positions), _ptr(slot_mapping), _ptr(q),
+            _ptr(k_cache), _ptr(v_cache), _code(self.act_dtype), T, Hq, Hkv, dim, vdim, P, page, self._stream()))
+        return q
+
+    def head_gate_(self, o, gate, gate_col, num_heads, head_dim):
+        self._on_device(o, gate)
+        T = o.shape[0]
+        if tuple(o.shape) != (T, num_heads * head_dim) or not o.is_contiguous():
+            raise ValueError(f"head_gate_: o {tuple(o.shape)} for {num_heads} heads of {head_dim}")
+        gp = self._f32_columns(gate, gate_col, num_heads, "head_gate_: gate")
+        if gate.shape[0] != T:
+            raise ValueError("head_gate_: one gate row a token")
+        lib = self.lib("attention_prep")
+        library.check(lib, lib.mie_head_gate(_ptr(o), _code(o.dtype), gp, gate.stride(0), T, num_heads, head_dim, self._stream()))
+        return o
+
+    def delta_rule(self, sums, cols, num_heads, dim, w_decay, decay_bias, decay_scale, removal_bias, norm_weight, eps,
+                   state, step):
+        self._on_device(sums, w_decay, decay_bias, removal_bias, norm_weight, state)
+        H, d, T = num_heads, dim, sums.shape[0]
+        n = H * d
+        if w_decay.dim() != 2 or w_decay.shape[0] != n:
+            raise ValueError(f"delta_rule: decay matrix {tuple(w_decay.shape)} for {H} heads of {d}")
+        rank = w_decay.shape[1]
+        self._f32_vector(w_decay, n * rank, "delta_rule: decay matrix")
+        for name in ("r", "k", "v", "g", "a"):
+            self._f32_columns(sums, cols[name], n, f"delta_rule: {name}")
+        self._f32_columns(sums, cols["w"], rank, "delta_rule: the decay's inner activations")
+        for name, t in (("decay_bias", decay_bias), ("removal_bias", removal_bias), ("norm_weight", norm_weight)):
+            self._f32_vector(t, n, f"delta_rule: {name}")
+        if state.dtype != torch.float32 or tuple(state.shape[1:]) != (H, d, d) or not state.is_contiguous():
+            raise ValueError(f"delta_rule: state {tuple(state.shape)} for {H} heads of {d} x {d}")
+        self._check_rows("delta_rule", step, T)
+        if int(step.host["state_slots"].max()) >= state.shape[0]:
+            raise ValueError("delta_rule: a state slot beyond the state's slots")
+        out = torch.empty((T, n), dtype=self.act_dtype, device=sums.device)
+        prep = torch.empty((T, 3 * n), dtype=torch.float32, device=sums.device)
+        lib = self.lib("delta_rule")
+        library.check(lib, lib.mie_delta_rule(
+            _ptr(sums), sums.stride(0), cols["r"], cols["k"], cols["v"], cols["g"], cols["a"], cols["w"], _ptr(w_decay), rank,
+            _ptr(decay_bias), float(decay_scale), _ptr(removal_bias), _ptr(norm_weight), float(eps), _ptr(state),
+            _ptr(step.row_start), _ptr(step.state_slots), _ptr(prep), _ptr(out), _code(out.dtype), T, step.num_rows, H, d,
+            self._stream()))
+        return out
+
+    def normed_sum_add(self, stream, ys, weights, eps, scale):
+        self._on_device(stream, *ys, *weights)
+        if stream.dtype != torch.float32 or stream.dim() != 2 or not stream.is_contiguous():
+            raise ValueError("normed_sum_add: the stream must be contiguous float32 [T, width]")
+        T, W = stream.shape
+        if not 1 <= len(ys) <= 2 or len(weights) != len(ys):
+            raise ValueError("normed_sum_add: one or two branch outputs, a weight each")
+        for y, w in zip(ys, weights):
+            if y.dtype != torch.float32 or tuple(y.shape) != (T, W) or not y.is_contiguous():
+                raise ValueError(f"normed_sum_add: a branch output {tuple(y.shape)} {y.dtype}; contiguous float32 {(T, W)} expected")
+            self._f32_vector(w, W, "normed_sum_add: weight")
+        lib = self.lib("embed_norm")
+        library.check(lib, lib.mie_normed_sum_add(_ptr(stream), _ptr(ys[0]), _ptr(weights[0]), _ptr(ys[1]) if len(ys) > 1 else None,
+                                                  _ptr(weights[1]) if len(ys) > 1 else None, T, W, float(eps), float(scale),
+                                                  self._stream()))
+        return stream
+
     def linear_rotary_kv_store(self, x, w_qkv, positions, cos, sin, rotary_dim, num_q_heads, num_kv_heads, head_dim,
                                k_cache, v_cache, slot_mapping, for_attention: bool = False):
         Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
@@ -867,11 +987,12 @@ class HipBackend(KernelBackend):
         return out
 
     def paged_attention(self, qkv, num_q_heads, num_kv_heads, head_dim, k_cache, v_cache, group, step, scale,
-                        window, force_generic: bool = False, num_splits: int | None = None):
+                        window, sink=None, force_generic: bool = False, num_splits: int | None = None):
         Hq, Hkv, D = num_q_heads, num_kv_heads, head_dim
+        has_sink, sink = int(sink is not None), float(sink or 0.0)
         if isinstance(qkv, ProjectionSums):
             out = self._decode_attention_from_sums(qkv, Hq, Hkv, D, k_cache, v_cache, group, step, scale, window,
-                                                   force_generic or num_splits is not None)
+                                                   force_generic or num_splits is not None or bool(has_sink))
             if out is not None:
                 return out
             qkv = qkv.finish()
@@ -894,10 +1015,13 @@ class HipBackend(KernelBackend):
             if splits > 1:
                 o_part = torch.empty((done, Hq, splits, D), dtype=torch.float32, device=qkv.device)
                 lse_part = torch.empty((done, Hq, splits), dtype=torch.float32, device=qkv.device)
-            library.check(lib, lib.mie_decode_attention(
-                _ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(o_part), _ptr(lse_part),
-                _ptr(bt), bt.shape[1], _ptr(step.positions), done, Hq, Hkv, D, page, float(scale), int(window or 0),
-                partition, splits, self._stream()))
+            args = (_ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(o_part), _ptr(lse_part),
+                    _ptr(bt), bt.shape[1], _ptr(step.positions), done, Hq, Hkv, D, page, float(scale), int(window or 0),
+                    partition, splits)
+            if has_sink:
+                library.check(lib, lib.mie_decode_attention_sink(*args, sink, self._stream()))
+            else:
+                library.check(lib, lib.mie_decode_attention(*args, self._stream()))
         if done < T and qkv.dtype == torch.bfloat16 and not force_generic:
             # rows of several tokens: matrix-core kernel over their own and earlier portions' keys
             for name, t, n in (("row_start", step.row_start, step.num_rows + 1),
@@ -905,11 +1029,14 @@ class HipBackend(KernelBackend):
                 if t is None or t.dtype != torch.int32 or t.shape[0] < n or not t.is_contiguous():
                     raise ValueError(f"paged_attention: {name} must be contiguous int32 [{n}]")
             lib = self.lib("prefill_attention_bf16", (f"-DHEAD_DIM={D}",))
-            library.check(lib, lib.mie_prefill_attention(
-                _ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(bt), bt.shape[1],
-                _ptr(step.row_start), _ptr(step.row_position), step.num_decode_rows,
-                step.num_rows - step.num_decode_rows, step.max_row_tokens, Hq, Hkv, D, page, float(scale),
-                int(window or 0), self._stream()))
+            args = (_ptr(qkv), qkv.stride(0), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(bt), bt.shape[1],
+                    _ptr(step.row_start), _ptr(step.row_position), step.num_decode_rows,
+                    step.num_rows - step.num_decode_rows, step.max_row_tokens, Hq, Hkv, D, page, float(scale),
+                    int(window or 0))
+            if has_sink:
+                library.check(lib, lib.mie_prefill_attention_sink(*args, sink, self._stream()))
+            else:
+                library.check(lib, lib.mie_prefill_attention(*args, self._stream()))
             done = T
         if done < T:
             lib = self.lib("attention")
@@ -918,7 +1045,7 @@ class HipBackend(KernelBackend):
                 c_void_p(qkv.data_ptr() + done * qkv.stride(0) * esz), qkv.stride(0), _ptr(k_cache), _ptr(v_cache),
                 c_void_p(out.data_ptr() + done * Hq * D * esz), _code(qkv.dtype), _ptr(bt), bt.shape[1],
                 c_void_p(step.token_row.data_ptr() + done * 4), c_void_p(step.positions.data_ptr() + done * 4),
-                T - done, Hq, Hkv, D, page, float(scale), int(window or 0), self._stream()))
+                T - done, Hq, Hkv, D, page, float(scale), int(window or 0), has_sink, sink, self._stream()))
         return out
 
     def sample(self, logits, temperatures, seeds, counters, out=None):

@@ -15,6 +15,7 @@ register_kernel_module("embed_norm", {
     "mie_branch_norm_add": [P, I, P, P, I, P, I, I, I, F, P],
     "mie_rmsnorm_columns": [P, L, P, I, P, I, I, I, F, P],
     "mie_scale": [P, L, F, P],
+    "mie_normed_sum_add": [P, P, P, P, P, I, I, F, F, P],
 })
 register_kernel_module("rope_kv", {
     "mie_rotary_kv_store": [P, I, L, P, P, P, I, I, I, I, P, P, P, I, I, P],
@@ -39,9 +40,17 @@ register_kernel_module("recurrence", {
     "mie_causal_conv": [P, L, P, P, P, P, P, P, P, P, I, I, I, P],
     "mie_rglru_scan": [P, P, P, P, L, P, P, L, P, P, P, P, P, P, I, I, I, I, F, P],
     "mie_rglru_scan_chunked": [P, P, P, P, L, P, P, L, P, P, P, P, P, P, I, I, I, I, F, I, I, P, P, P, P],
+    "mie_residual_conv": [P, P, P, P, P, P, P, I, I, I, I, I, P],
+})
+register_kernel_module("attention_prep", {
+    "mie_qkv_finish": [P, L, I, I, I, P, P, F, P, I, I, P, P, P, P, P, P, I, I, I, I, I, I, I, I, P],
+    "mie_head_gate": [P, I, P, L, I, I, I, P],
+})
+register_kernel_module("delta_rule", {
+    "mie_delta_rule": [P, L, I, I, I, I, I, I, P, I, P, F, P, P, F, P, P, P, P, P, I, I, I, I, I, P],
 })
 register_kernel_module("attention", {
-    "mie_paged_attention": [P, L, P, P, P, I, P, I, P, P, I, I, I, I, I, F, I, P],
+    "mie_paged_attention": [P, L, P, P, P, I, P, I, P, P, I, I, I, I, I, F, I, I, F, P],
 })
 register_kernel_module("sampling", {
     "mie_sample": [P, L, P, P, P, P, I, I, P],
@@ -60,6 +69,7 @@ register_kernel_module("gemm_mid_bf16", {
 })
 register_kernel_module("attention_bf16", {
     "mie_decode_attention": [P, L, P, P, P, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P],
+    "mie_decode_attention_sink": [P, L, P, P, P, P, P, P, I, P, I, I, I, I, I, F, I, I, I, F, P],
     "mie_decode_attention_from_sums": [P, I, L, L, P, P, P, P, P, P, P, I, P, I, I, I, I, I, F, I, I, P],
     "mie_decode_attention_static": [P, L, P, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P],
     "mie_decode_attention_static_setup": [],
@@ -71,6 +81,7 @@ register_kernel_module("attention_bf16", {
 # every key block for the sake of the (rare) rescaling.
 register_kernel_module("prefill_attention_bf16", {
     "mie_prefill_attention": [P, L, P, P, P, P, I, P, P, I, I, I, I, I, I, I, F, I, P],
+    "mie_prefill_attention_sink": [P, L, P, P, P, P, I, P, P, I, I, I, I, I, I, I, F, I, F, P],
 }, variants=_head_variants, flags=["-mllvm", "-amdgpu-mfma-vgpr-form"])
 # lt_gemm: host code only, the engine's own way into the library's matrix products (hipBLASLt) with the choice of
 # kernel per shape kept here.

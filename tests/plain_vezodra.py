@@ -74,7 +74,7 @@ def softmax_attention(q, k, v, scale, window=None, sink=None):
     return torch.einsum("hij,jhd->ihd", e / denom, v.repeat_interleave(rep, 1))
 
 
-def sink_attention(w, p, m, h, positions):
+def sink_attention(w, p, m, h, positions, sink=0.0):
     """Mixer 'attention': values are the keys as projected (before they turn), a per-head temperature on the
     scores, a sink of score 0, a sigmoid gate per head on the output."""
     n, H, G, d = h.shape[0], m["heads"], m["kv_heads"], m["dim"]
@@ -82,7 +82,7 @@ def sink_attention(w, p, m, h, positions):
     k = (h @ w[p + "k"].T).view(n, G, d)
     v = k
     q, k = rotate(q, positions, m["rot"], "interleaved"), rotate(k, positions, m["rot"], "interleaved")
-    o = softmax_attention(q, k, v, m["scale"] * w[p + "temp"], sink=0.0)
+    o = softmax_attention(q, k, v, m["scale"] * w[p + "temp"], sink=sink)
     o = o * torch.sigmoid(h @ w[p + "g"].T)[:, :, None]
     return o.reshape(n, H * d) @ w[p + "o"].T
 
@@ -140,16 +140,20 @@ def run_order(config):
     return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
 
 
-def forward(config, weights, ids, streams=None):
+def forward(config, weights, ids, streams=None, sink=0.0):
+    """``sink``: the score of the 'attention' mixer's sink (the design fixes 0; None leaves it out, for tests that
+    show that it matters)."""
     w = {k: (v.double() if v.is_floating_point() else v) for k, v in weights.items()}
     eps = config["norm"]["eps"]
     positions = torch.arange(len(ids))
     s = w["embed"][torch.tensor(ids)]
     for i in run_order(config):
         layer, p = config["layers"][i], f"l{i}."
-        h = input_conv(rms_norm(s, w[p + "norm1"], eps), w[p + "canon1"])
+        h = rms_norm(s, w[p + "norm1"], eps)
+        if config.get("canon") is not None:
+            h = input_conv(h, w[p + "canon1"])
         if layer["type"] == "attention":
-            branch = sink_attention(w, p + "mix.", layer["mixer"], h, positions)
+            branch = sink_attention(w, p + "mix.", layer["mixer"], h, positions, sink)
         elif layer["type"] == "parallel":
             branch = parallel_mixer(w, p + "mix.", layer["mixer"], h, positions, eps)
         else:
