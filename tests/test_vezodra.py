@@ -337,7 +337,8 @@ def edge_runs(device):
     got = {k: v.cpu() for k, v in trace_util.run_on_runner(runner, trace_util.decode_tail({"x": toks}, 30)).items()}
     trace_util.compare(got, {"x": want}, F32_TOL, "sink")
     moved = (plain.forward(raw, w, toks, sink=None) - want).abs().amax(-1) / float(want.abs().max())
-    assert float(moved.min()) > 10 * F32_TOL, "leaving the sink out must show at every position, the first included"
+    assert float(moved[0]) > 30 * F32_TOL and float(moved[:8].min()) > 3 * F32_TOL and float(moved[30:].max()) > 3 * F32_TOL, \
+        "leaving the sink out must show, at the first position above all (one key, and the sink beside it)"
 
 
 def test_window_edges_and_the_sink():
@@ -571,11 +572,11 @@ def test_attention_kernels_with_a_sink(hip, dtype):
     """The three attention kernels (32-bit, matrix-core decode with and without splits, matrix-core prompt portions)
     with one more term in the denominator; scores spread so that the term matters (and so that it is sometimes the
     largest)."""
-    from test_kernels_gpu import make_case
+    from test_kernels_gpu import paged_setup
     ops = hip[dtype]
-    for (Hq, Hkv, D, lens, starts, window, sink) in ((4, 2, 32, [1, 1, 1], [300, 17, 0], None, 0.0), (6, 3, 96, [40, 1, 7], [100, 5, 0], None, 0.0),
-                                                     (2, 1, 64, [1, 1], [2000, 900], None, 1.5), (4, 4, 16, [33, 2], [0, 64], 20, -0.5)):
-        q, kc, vc, group, step = make_case(dtype, Hq, Hkv, D, lens, starts, seed=len(lens) + D)
+    for (Hq, Hkv, D, ctx, lens, window, sink) in ((4, 2, 32, [3, 18, 1], [1, 1, 1], None, -0.5), (6, 3, 96, [6, 140, 7], [1, 40, 7], None, 0.0),
+                                                  (2, 1, 64, [2001, 901], [1, 1], None, 8.0), (4, 4, 16, [33, 66], [33, 2], 20, 3.0)):
+        q, kc, vc, group, step = paged_setup(ctx, lens, Hq, Hkv, D, 16, dtype)
         scale = 2.0 / math.sqrt(D)
         expect = ref.ref_paged_attention(q, Hq, Hkv, D, kc, vc, group.block_tables, step.token_row, step.positions, scale, window,
                                          torch.float64, sink=sink)
@@ -644,7 +645,7 @@ def test_command_line_and_trace_runner(tmp_path):
         return proc
 
     cli = [sys.executable, "-m", "mini_inference_engine_amd"]
-    run(cli + ["random-model", "--shape", "vezodra-tiny", "--seed", "3", "--dtype", "float32", "--std", "0.2", "--out", folder])
+    run(cli + ["random-model", "--shape", "vezodra-tiny", "--seed", "3", "--dtype", "float32", "--out", folder])
     raw = json.load(open(os.path.join(folder, "config.json")))
     weights = load_file(os.path.join(folder, "model.safetensors"))
     assert raw["architecture"] == "Vezodra" and len(raw["layers"]) == 3 and raw["loop"]["times"] == 2
