@@ -3,8 +3,8 @@ Llama-2-7B or Llama-3-8B), random weights.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--shape tinyllama] [--context N] [--layers L]
     python bench.py --kernels [--shape ...] [--batch 8] [--context N]     each dominant kernel alone
-    python bench.py --design zifelorn [--design-sizes 1024,2048] [--layers R] [--batch 8] [--context 1024]
-                                                 Zifelorn beside Llama at equal layer sizes (R runs of four layers)
+    python bench.py --design zifelorn|vezodra [--design-sizes 1024,2048] [--layers R] [--batch 8] [--context 1024]
+                                                 that design beside Llama at equal layer sizes (R runs of its layers)
 
 A step is one decode step of the engine (schedule, batch, captured forward, sampling,
 bookkeeping: LLMEngine.step, the call a user's loop makes; it starts a step and reads the tokens
@@ -439,20 +439,36 @@ DESIGN_SIZES = {
 }
 
 
-def design_configs(size: str, repeats: int):
-    from mini_inference_engine_amd.config import LlamaConfig, ZifelornConfig
-    from mini_inference_engine_amd.models.zifelorn import _shape
-    z = DESIGN_SIZES[size]
-    zcfg = ZifelornConfig.from_dict(_shape(repeats=repeats, **z))
+# Vezodra layer sizes of the same widths: a run of three layers is window attention beside the delta rule, attention
+# with a sink, window attention beside the delta rule, each with the dense feed-forward; every layer runs once.
+VEZODRA_SIZES = {
+    "1024": dict(vocab=32000, width=1024, ff=2816, heads=16, kv_heads=4, dim=64, window=1024, rec_heads=16, rec_dim=64, rank=64,
+                 sink_heads=8, sink_kv_heads=2, sink_dim=128),
+    "2048": dict(vocab=32000, width=2048, ff=5632, heads=32, kv_heads=8, dim=64, window=1024, rec_heads=32, rec_dim=64, rank=64,
+                 sink_heads=16, sink_kv_heads=4, sink_dim=128),
+}
+
+
+def design_configs(design: str, size: str, repeats: int):
+    """(the design's configuration, Llama's of the same width, head count, feed-forward size, vocabulary and layer count)."""
+    from mini_inference_engine_amd.config import LlamaConfig, VezodraConfig, ZifelornConfig
+    if design == "vezodra":
+        from mini_inference_engine_amd.models.vezodra import _shape
+        z = VEZODRA_SIZES[size]
+        cfg, layers = VezodraConfig.from_dict(_shape(repeats=repeats, times=1, **z)), 3 * repeats
+    else:
+        from mini_inference_engine_amd.models.zifelorn import _shape
+        z = DESIGN_SIZES[size]
+        cfg, layers = ZifelornConfig.from_dict(_shape(repeats=repeats, **z)), 4 * repeats
     lcfg = LlamaConfig.from_dict(dict(
-        vocab_size=z["vocab"], hidden_size=z["width"], intermediate_size=z["ff"], num_hidden_layers=4 * repeats,
+        vocab_size=z["vocab"], hidden_size=z["width"], intermediate_size=z["ff"], num_hidden_layers=layers,
         num_attention_heads=z["heads"], num_key_value_heads=max(1, z["heads"] // 4), head_dim=z["width"] // z["heads"],
         rms_norm_eps=1e-5, rope_theta=10000.0, max_position_embeddings=8192, tie_word_embeddings=True))
-    return zcfg, lcfg
+    return cfg, lcfg, layers
 
 
 def measure_designs(args) -> int:
-    """Decode (batch ``--batch``, contexts of ``--context``) and a 2,048-token prefill of Zifelorn beside Llama at
+    """Decode (batch ``--batch``, contexts of ``--context``) and a 2,048-token prefill of the design beside Llama at
     equal sizes, through LLMEngine.step, random weights; one JSON line."""
     import torch
     from mini_inference_engine_amd import LLMEngine
@@ -463,7 +479,8 @@ def measure_designs(args) -> int:
            "batch": args.batch, "context": context, "steps": args.steps, "sizes": {}}
     for size in (args.design_sizes.split(",") if args.design_sizes else DESIGN_SIZES):
         row = {}
-        for name, cfg in zip(("zifelorn", "llama"), design_configs(size, args.layers or 1)):
+        dcfg, lcfg, layers = design_configs(args.design, size, args.layers or 1)
+        for name, cfg in ((args.design, dcfg), ("llama", lcfg)):
             weights = random_tensors(cfg, args.seed, torch.bfloat16, std=0.02, device="cuda")
             pages = args.batch * (-(-max(context, 2048) // args.block_size)) + 1 + 64
             ecfg = EngineConfig(block_size=args.block_size, max_num_seqs=args.batch, max_num_batched_tokens=2048,
@@ -473,7 +490,7 @@ def measure_designs(args) -> int:
             eng.model_cfg_vocab = getattr(cfg, "vocab_size", None) or cfg.vocab
             dt, captured, ctx = measure_decode(eng, args.batch, context, args.steps, args.warmup, args.seed, vocab=eng.model_cfg_vocab)
             t = measure_prefill(eng, 2048, args.seed + 100, vocab=eng.model_cfg_vocab)
-            row[name] = {"layers": 4 * (args.layers or 1), "decode_tok_s": round(args.batch * args.steps / dt, 1),
+            row[name] = {"layers": layers, "decode_tok_s": round(args.batch * args.steps / dt, 1),
                          "decode_ms_per_step": round(dt / args.steps * 1e3, 4), "captured_steps": captured,
                          "prefill_2048_tok_s": round(2048 / t, 1), "prefill_ms": round(t * 1e3, 3),
                          "weight_MB": round(eng.runner.model.weight_bytes() / 1e6, 1)}
@@ -486,8 +503,8 @@ def measure_designs(args) -> int:
 
 def main() -> int:
     ap = argparse.ArgumentParser()
-    ap.add_argument("--design", choices=["zifelorn"], default=None,
-                    help="instead of the default workload: Zifelorn beside Llama at equal layer sizes (decode and prefill)")
+    ap.add_argument("--design", choices=["zifelorn", "vezodra"], default=None,
+                    help="instead of the default workload: that design beside Llama at equal layer sizes (decode and prefill)")
     ap.add_argument("--design-sizes", default=None, help="comma-separated widths of --design (default: all of 1024, 2048)")
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)

@@ -368,6 +368,95 @@ MIE_EXPORT int mie_normed_sum_add(float* stream, const float* a, const float* wa
   return 0;
 }
 
+// ---- two norms of the same stream and a short convolution on the first, in one pass:
+//   h = x * rstd(x) * w1;  xm[t] = h[t] + sum_k taps[:, k] h[t - (K - 1 - k)]  (a row's earlier tokens; before its first
+//   token the K - 1 inputs kept in tail[slot]);  y = x * rstd(x) * w2 (w2 null: none).  One workgroup a token: it
+//   takes the root mean square of its own row and of the K - 1 rows before it in the step, and leaves its own in
+//   rstd[t] for norm_conv_tail_kernel, which afterwards moves every row's last K - 1 inputs into tail[slot] (a thread
+//   a (row, channel), reads ahead of writes).
+constexpr int CONV_MAX_TAPS = 8;
+
+template <typename TO>
+__global__ void __launch_bounds__(NORM_THREADS)
+norm_pair_conv_kernel(const float* __restrict__ stream, const float* __restrict__ w1, const float* __restrict__ w2,
+                      const float* __restrict__ taps, const float* __restrict__ tail, const int* __restrict__ token_row,
+                      const int* __restrict__ row_start, const int* __restrict__ slots, TO* __restrict__ xm,
+                      TO* __restrict__ y, float* __restrict__ rstd_out, int width, int K, float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  const int r = token_row[t], j = t - row_start[r];
+  const int have = j < K - 1 ? j : K - 1;            // rows before this one that are in the step
+  float ss[CONV_MAX_TAPS];
+#pragma unroll
+  for (int b = 0; b < CONV_MAX_TAPS; ++b) ss[b] = 0.f;
+  for (int i = threadIdx.x; i < width; i += NORM_THREADS) {
+#pragma unroll
+    for (int b = 0; b < CONV_MAX_TAPS; ++b)
+      if (b <= have) {
+        const float v = stream[(size_t)(t - b) * width + i];
+        ss[b] = fmaf(v, v, ss[b]);
+      }
+  }
+  float rstd[CONV_MAX_TAPS];
+#pragma unroll
+  for (int b = 0; b < CONV_MAX_TAPS; ++b)
+    rstd[b] = b <= have ? 1.0f / sqrtf(block_sum(ss[b], scratch) / (float)width + eps) : 0.f;    // ``have`` is the workgroup's
+  if (threadIdx.x == 0) rstd_out[t] = rstd[0];
+  const float* tl = tail + (size_t)slots[r] * (K > 1 ? K - 1 : 1) * width;
+  for (int i = threadIdx.x; i < width; i += NORM_THREADS) {
+    const float g = w1[i];
+    const float own = stream[(size_t)t * width + i];
+    float acc = own * rstd[0] * g;
+#pragma unroll
+    for (int b = 0; b < CONV_MAX_TAPS; ++b)
+      if (b < K) {
+        const float h = b <= have ? stream[(size_t)(t - b) * width + i] * rstd[b] * g : tl[(size_t)(K - 1 + j - b) * width + i];
+        acc = fmaf(taps[(size_t)i * K + (K - 1 - b)], h, acc);
+      }
+    xm[(size_t)t * width + i] = from_float<TO>(acc);
+    if (w2) y[(size_t)t * width + i] = from_float<TO>(own * rstd[0] * w2[i]);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+norm_conv_tail_kernel(const float* __restrict__ stream, const float* __restrict__ w1, const float* __restrict__ rstd,
+                      float* __restrict__ tail, const int* __restrict__ row_start, const int* __restrict__ slots, int width,
+                      int K) {
+  const int r = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= width) return;
+  const int a0 = row_start[r], n = row_start[r + 1] - a0, keep = K - 1;
+  float* tl = tail + (size_t)slots[r] * keep * width;
+  for (int i = 0; i < keep; ++i) {
+    const int src = n + i;                     // place in the joined sequence of keep + n inputs
+    const int tok = a0 + src - keep;
+    tl[(size_t)i * width + c] = src < keep ? tl[(size_t)src * width + c] : stream[(size_t)tok * width + c] * rstd[tok] * w1[c];
+  }
+}
+
+// stream [tokens, width] float32; w1, w2 (or null), taps [width, K] float32; tail [slots, max(1, K - 1), width] float32;
+// xm, y [tokens, width] of out_dtype; rstd: scratch of tokens floats.
+MIE_EXPORT int mie_norm_pair_conv(const float* stream, const float* w1, const float* w2, const float* taps, float* tail,
+                                  const int* token_row, const int* row_start, const int* slots, void* xm, void* y, int out_dtype,
+                                  float* rstd, int tokens, int rows, int width, int K, float eps, hipStream_t s) {
+  if (tokens <= 0 || rows <= 0) return 0;
+  if (width <= 0 || K < 1 || K > CONV_MAX_TAPS) MIE_FAIL("norm_pair_conv: width %d, %d taps (1 to %d)", width, K, CONV_MAX_TAPS);
+  if (!stream || !w1 || !taps || !tail || !xm || !rstd || (w2 && !y)) MIE_FAIL("norm_pair_conv: a missing operand");
+  if (out_dtype == MIE_F32)
+    hipLaunchKernelGGL(norm_pair_conv_kernel<float>, dim3(tokens), dim3(NORM_THREADS), 0, s, stream, w1, w2, taps, tail, token_row,
+                       row_start, slots, (float*)xm, (float*)y, rstd, width, K, eps);
+  else if (out_dtype == MIE_BF16)
+    hipLaunchKernelGGL(norm_pair_conv_kernel<bf16>, dim3(tokens), dim3(NORM_THREADS), 0, s, stream, w1, w2, taps, tail, token_row,
+                       row_start, slots, (bf16*)xm, (bf16*)y, rstd, width, K, eps);
+  else MIE_FAIL("norm_pair_conv: out dtype code %d", out_dtype);
+  MIE_CHECK_LAUNCH("norm_pair_conv");
+  if (K > 1) {
+    hipLaunchKernelGGL(norm_conv_tail_kernel, dim3(rows, (width + 255) / 256), dim3(256), 0, s, stream, w1, rstd, tail, row_start,
+                       slots, width, K);
+    MIE_CHECK_LAUNCH("norm_pair_conv (tail)");
+  }
+  return 0;
+}
+
 // ---- t *= factor
 __global__ void scale_kernel(float* __restrict__ t, size_t n, float factor) {
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) t[i] *= factor;

@@ -177,6 +177,15 @@ class KernelBackend:
         including this step's.  All float32 -> [T, C] in ``out_dtype`` (default: the activation dtype)."""
         raise NotImplementedError
 
+    def norm_pair_conv(self, stream, w_first, w_second, eps, taps, tail, step):
+        """Two RMS norms of the same float32 stream [T, width] and the short convolution of ``residual_conv`` on the
+        first: x = residual_conv(rmsnorm(stream) * w_first), y = rmsnorm(stream) * w_second (None: no second norm),
+        both in the activation dtype; ``tail`` moves on.  -> (x, y).  A backend may do it in one pass."""
+        import torch
+        h = self.add_rmsnorm(None, stream, w_first, eps, out_dtype=torch.float32)
+        x = self.residual_conv(h, taps, tail, step)
+        return x, (None if w_second is None else self.add_rmsnorm(None, stream, w_second, eps))
+
     def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
                    layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None):
         """What lies between a q/k/v projection's float32 sums [T, *] and attention, in 32-bit: queries are columns

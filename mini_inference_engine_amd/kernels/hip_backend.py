@@ -701,7 +701,40 @@ class HipBackend(KernelBackend):
                                                  self._stream()))
         return y
 
+    NORM_CONV_MAX_TAPS = 8
+
+    def norm_pair_conv(self, stream, w_first, w_second, eps, taps, tail, step):
+        self._on_device(stream, w_first, w_second, taps, tail)
+        K = taps.shape[1] if taps.dim() == 2 else 0
+        plain = lambda t: t is None or (t.dtype == torch.float32 and t.is_contiguous())      # noqa: E731
+        if not 1 <= K <= self.NORM_CONV_MAX_TAPS or not (plain(w_first) and plain(w_second)):
+            return super().norm_pair_conv(stream, w_first, w_second, eps, taps, tail, step)
+        if stream.dtype != torch.float32 or stream.dim() != 2 or not stream.is_contiguous():
+            raise ValueError("norm_pair_conv: the stream must be contiguous float32 [T, width]")
+        T, W = stream.shape
+        self._f32_vector(w_first, W, "norm_pair_conv: first weight")
+        if w_second is not None:
+            self._f32_vector(w_second, W, "norm_pair_conv: second weight")
+        if taps.shape[0] != W:
+            raise ValueError(f"norm_pair_conv: taps {tuple(taps.shape)} for width {W}")
+        self._f32_vector(taps, W * K, "norm_pair_conv: taps")
+        if tail.dtype != torch.float32 or tuple(tail.shape[1:]) != (max(1, K - 1), W) or not tail.is_contiguous():
+            raise ValueError(f"norm_pair_conv: tail {tuple(tail.shape)} for {K} taps of width {W}")
+        self._check_rows("norm_pair_conv", step, T)
+        if int(step.host["state_slots"].max()) >= tail.shape[0]:
+            raise ValueError("norm_pair_conv: a state slot beyond the tail's slots")
+        x = torch.empty((T, W), dtype=self.act_dtype, device=stream.device)
+        y = torch.empty((T, W), dtype=self.act_dtype, device=stream.device) if w_second is not None else None
+        rstd = torch.empty(T, dtype=torch.float32, device=stream.device)
+        lib = self.lib("embed_norm")
+        library.check(lib, lib.mie_norm_pair_conv(_ptr(stream), _ptr(w_first), _ptr(w_second), _ptr(taps), _ptr(tail),
+                                                  _ptr(step.token_row), _ptr(step.row_start), _ptr(step.state_slots), _ptr(x),
+                                                  _ptr(y), _code(self.act_dtype), _ptr(rstd), T, step.num_rows, W, K, float(eps),
+                                                  self._stream()))
+        return x, y
+
     LAYOUTS = {"interleaved": 0, "half": 1}
+    DELTA_CHUNK = 64         # tokens a chunk of the delta rule's scan; rows up to this long run whole
 
     def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
                    layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None):
@@ -773,12 +806,20 @@ class HipBackend(KernelBackend):
             raise ValueError("delta_rule: a state slot beyond the state's slots")
         out = torch.empty((T, n), dtype=self.act_dtype, device=sums.device)
         prep = torch.empty((T, 3 * n), dtype=torch.float32, device=sums.device)
+        longest = int(getattr(step, "max_row_tokens", 0) or (step.host["row_start"][1:] - step.host["row_start"][:-1]).max())
+        chunk, chunks, summaries, starts = 0, 0, None, None
+        if longest > self.DELTA_CHUNK and not self.true_fp32:
+            # rows of many tokens: chunks side by side (whether a step takes this path depends on its longest row alone;
+            # the two paths differ by the rounding of the fold over whole chunks, so the 32-bit mode keeps to one)
+            chunk, chunks = self.DELTA_CHUNK, -(-longest // self.DELTA_CHUNK)
+            scratch = torch.empty((3, step.num_rows * chunks * H, d, d), dtype=torch.float32, device=sums.device)
+            summaries, starts = scratch[:2], scratch[2]
         lib = self.lib("delta_rule")
         library.check(lib, lib.mie_delta_rule(
             _ptr(sums), sums.stride(0), cols["r"], cols["k"], cols["v"], cols["g"], cols["a"], cols["w"], _ptr(w_decay), rank,
             _ptr(decay_bias), float(decay_scale), _ptr(removal_bias), _ptr(norm_weight), float(eps), _ptr(state),
             _ptr(step.row_start), _ptr(step.state_slots), _ptr(prep), _ptr(out), _code(out.dtype), T, step.num_rows, H, d,
-            self._stream()))
+            chunk, chunks, _ptr(summaries), _ptr(starts), self._stream()))
         return out
 
     def normed_sum_add(self, stream, ys, weights, eps, scale):

@@ -16,6 +16,7 @@ register_kernel_module("embed_norm", {
     "mie_rmsnorm_columns": [P, L, P, I, P, I, I, I, F, P],
     "mie_scale": [P, L, F, P],
     "mie_normed_sum_add": [P, P, P, P, P, I, I, F, F, P],
+    "mie_norm_pair_conv": [P, P, P, P, P, P, P, P, P, P, I, P, I, I, I, I, F, P],
 })
 register_kernel_module("rope_kv", {
     "mie_rotary_kv_store": [P, I, L, P, P, P, I, I, I, I, P, P, P, I, I, P],
@@ -47,7 +48,7 @@ register_kernel_module("attention_prep", {
     "mie_head_gate": [P, I, P, L, I, I, I, P],
 })
 register_kernel_module("delta_rule", {
-    "mie_delta_rule": [P, L, I, I, I, I, I, I, P, I, P, F, P, P, F, P, P, P, P, P, I, I, I, I, I, P],
+    "mie_delta_rule": [P, L, I, I, I, I, I, I, P, I, P, F, P, P, F, P, P, P, P, P, I, I, I, I, I, I, I, P, P, P],
 })
 register_kernel_module("attention", {
     "mie_paged_attention": [P, L, P, P, P, I, P, I, P, P, I, I, I, I, I, F, I, I, F, P],

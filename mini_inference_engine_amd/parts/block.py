@@ -108,6 +108,11 @@ class ParallelBlock(Block):
             return self.mixer.cache_requirement()
         return CombinedCache([("mixer", self.mixer.cache_requirement()), ("conv", self.input_conv.cache_requirement())])
 
+    def prepare(self, device, dtype):
+        # the norms' weights in 32-bit for the pass that makes both norms at once
+        self._w_mixer = self.norm_mixer.weight.float().contiguous()
+        self._w_ff = None if self.norm_feed_forward is None else self.norm_feed_forward.weight.float().contiguous()
+
     def forward(self, h, residual, step, cache, next_norm=None):
         import torch
         ops = self.ops
@@ -117,14 +122,16 @@ class ParallelBlock(Block):
             h = None
         if h is not None:
             residual.add_(h.float())
-        conv = self.input_conv
-        x = ops.add_rmsnorm(None, residual, self.norm_mixer.weight, self.norm_mixer.eps,
-                            out_dtype=torch.float32 if conv is not None else None)
-        if conv is not None:
-            x = conv.forward(x, step, cache.sub("conv"))
-        y = None
-        if self.feed_forward is not None:
-            y = ops.add_rmsnorm(None, residual, self.norm_feed_forward.weight, self.norm_feed_forward.eps)
+        conv, nm, nf = self.input_conv, self.norm_mixer, self.norm_feed_forward
+        if conv is not None and (nf is None or nf.eps == nm.eps):
+            # both norms divide by the same root mean square: one pass over the stream makes both, and the convolution
+            x, y = ops.norm_pair_conv(residual, self._w_mixer, None if nf is None else self._w_ff, nm.eps, conv.weight,
+                                      cache.sub("conv").tensors["tail"], step)
+        else:
+            x = ops.add_rmsnorm(None, residual, nm.weight, nm.eps, out_dtype=torch.float32 if conv is not None else None)
+            if conv is not None:
+                x = conv.forward(x, step, cache.sub("conv"))
+            y = None if nf is None else ops.add_rmsnorm(None, residual, nf.weight, nf.eps)
         sink = Sink(residual)
         a = self.mixer.forward(x, step, cache.sub("mixer") if conv is not None else cache, add_to=sink)
         if a is not None:

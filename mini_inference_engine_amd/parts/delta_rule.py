@@ -60,11 +60,15 @@ class DeltaRule(Mixer):
         for attr in ("w_decay", "decay_bias", "removal_bias", "norm"):
             setattr(self, attr, getattr(self, attr).float().contiguous())
 
-    def forward(self, x, step, cache, add_to=None):
+    def forward(self, x, step, cache, add_to=None, sums=None, base=0):
+        """``sums``: the float32 sums of a product that holds this part's ``w_in`` rows from column ``base`` on (a
+        caller that stacked several parts' input matrices); ``x`` is then not read."""
         import torch
         ops = self.ops
-        sums = ops.linear(x, self.w_in, out_dtype=torch.float32)
-        out = ops.delta_rule(sums, self.cols, self.num_heads, self.dim, self.w_decay, self.decay_bias, self.decay_scale,
+        if sums is None:
+            sums, base = ops.linear(x, self.w_in, out_dtype=torch.float32), 0
+        cols = self.cols if base == 0 else {k: v + base for k, v in self.cols.items()}
+        out = ops.delta_rule(sums, cols, self.num_heads, self.dim, self.w_decay, self.decay_bias, self.decay_scale,
                              self.removal_bias, self.norm, self.eps, cache.state, step)
         if add_to is None and self.float32_output:
             return ops.linear(out, self.w_o, out_dtype=torch.float32)

@@ -24,13 +24,30 @@ class SideBySide(Mixer):
         return CombinedCache([("left", self.left.cache_requirement()), ("right", self.right.cache_requirement())])
 
     def prepare(self, device, dtype):
+        import torch
         self.left_norm, self.right_norm = self.left_norm.float().contiguous(), self.right_norm.float().contiguous()
+        # Both sides read the same input: where each has one input matrix (``w_in``) and takes a product's sums, the
+        # two matrices are stacked and one product serves both.
+        self.w_in = None
+        for side in (self.left, self.right):
+            side.prepare(device, dtype)
+        wl, wr = getattr(self.left, "w_in", None), getattr(self.right, "w_in", None)
+        if wl is not None and wr is not None and wl.dtype == wr.dtype and wl.shape[1] == wr.shape[1]:
+            self.w_in = torch.cat([wl, wr]).contiguous()
+            self.right_base = wl.shape[0]
+            self.left.w_in = self.w_in[:wl.shape[0]]
+            self.right.w_in = self.w_in[wl.shape[0]:]
 
     def forward(self, x, step, cache, add_to=None):
         import torch
         ops = self.ops
-        yl = self.left.forward(x, step, cache.sub("left"))
-        yr = self.right.forward(x, step, cache.sub("right"))
+        if self.w_in is not None:
+            sums = ops.linear(x, self.w_in, out_dtype=torch.float32)
+            yl = self.left.forward(None, step, cache.sub("left"), sums=sums, base=0)
+            yr = self.right.forward(None, step, cache.sub("right"), sums=sums, base=self.right_base)
+        else:
+            yl = self.left.forward(x, step, cache.sub("left"))
+            yr = self.right.forward(x, step, cache.sub("right"))
         stream = getattr(add_to, "stream", add_to)
         if stream is None:
             stream = torch.zeros((yl.shape[0], self.width), dtype=torch.float32, device=yl.device)

@@ -93,22 +93,26 @@ class SoftmaxAttention(Mixer):
             if getattr(self, attr, None) is not None:
                 setattr(self, attr, getattr(self, attr).float().contiguous())
 
-    def forward(self, x, step, cache, add_to=None):
+    def forward(self, x, step, cache, add_to=None, sums=None, base=0):
+        """``sums``: the float32 sums of a product that holds this part's ``w_in`` rows from column ``base`` on (a
+        caller that stacked several parts' input matrices); ``x`` is then not read."""
         import torch
         ops, H, G, P = self.ops, self.num_heads, self.num_kv_heads, self.padded_dim
         if cache.k.shape[-1] != P:
             raise ValueError(f"the cache holds heads of {cache.k.shape[-1]} numbers; this layer's are {P}")
         group = step.groups[cache.group]
-        sums = ops.linear(x, self.w_in, out_dtype=torch.float32)
+        if sums is None:
+            sums, base = ops.linear(x, self.w_in, out_dtype=torch.float32), 0
         pos = self.position
-        q = ops.qkv_finish(sums, self.q_col, self.k_col, self.v_col, H, G, self.dim, self.vdim, P, step.positions,
+        q = ops.qkv_finish(sums, base + self.q_col, base + self.k_col, None if self.v_col is None else base + self.v_col,
+                           H, G, self.dim, self.vdim, P, step.positions,
                            pos.inv_freq if pos is not None else None, pos.layout if pos is not None else "half",
                            cache.k, cache.v, group.slot_mapping, q_norm=self.q_norm if self.qk_norm else None,
                            k_norm=self.k_norm if self.qk_norm else None, eps=self.eps,
                            q_head_scale=self.temperature if self.head_temperature else None)
         o = ops.paged_attention(q, H, G, P, cache.k, cache.v, group, step, self.scale, self.window, sink=self.sink)
         if self.head_gate:
-            o = ops.head_gate_(o, sums, self.gate_col, H, P)
+            o = ops.head_gate_(o, sums, base + self.gate_col, H, P)
         if add_to is None and self.float32_output:
             return ops.linear(o, self.w_o, out_dtype=torch.float32)
         return ops.linear(o, self.w_o, add_to=add_to)

@@ -495,6 +495,20 @@ def test_conv_and_joined_norm_kernels(hip, dtype):
         close(got, want, TOL[dtype], "conv")
         if K > 1:
             assert torch.equal(tail.cpu(), want_tail), "the tail holds the last inputs as they were given"
+        # the same behind two norms of one stream, in one pass
+        stream, w1, w2 = _rand((step.num_tokens, C), torch.float32, g, 2.0), _rand((C,), torch.float32, g) + 1, _rand((C,), torch.float32, g) + 1
+        tail2 = _rand((6, max(1, K - 1), C), torch.float32, g)
+        want_tail = tail2.cpu().clone()
+        hn = ref.ref_add_rmsnorm(None, stream.cpu(), w1.cpu(), 1e-5, torch.float32)
+        want_x = ref.ref_residual_conv(hn, taps.cpu(), want_tail, step.host["row_start"], step.host["state_slots"], dtype)
+        for second in (w2, None):
+            tl = tail2.clone()
+            x, y = ops.norm_pair_conv(stream, w1, second, 1e-5, taps, tl, step)
+            close(x, want_x, TOL[dtype], "norms and conv in one pass")
+            close(tl, want_tail, 3e-6, "tail behind the norm")
+            assert (y is None) == (second is None)
+            if y is not None:
+                close(y, ref.ref_add_rmsnorm(None, stream.cpu(), w2.cpu(), 1e-5, dtype), TOL[dtype], "second norm")
     for T, W in ((1, 64), (5, 70), (3, 4100)):
         stream = _rand((T, W), torch.float32, g)
         ys = [_rand((T, W), torch.float32, g, 3.0), _rand((T, W), torch.float32, g, 0.2)]
@@ -549,7 +563,9 @@ def test_attention_preparation_kernels(hip, dtype):
 def test_delta_rule_kernel(hip, dtype):
     ops, g = hip[dtype], torch.Generator().manual_seed(3)
     for (H, d, rank, lens, slots) in ((2, 16, 8, [1, 1, 9, 2, 70], [4, 1, 3, 5, 2]), (1, 32, 3, [5, 1], [1, 2]), (5, 12, 5, [3, 2, 40], [2, 3, 1]),
-                                      (3, 8, 5, [33], [5]), (2, 64, 16, [1, 20], [1, 2]), (1, 128, 4, [6], [3]), (1, 144, 4, [3, 1], [3, 1])):
+                                      (3, 8, 5, [33], [5]), (2, 64, 16, [1, 20], [1, 2]), (1, 128, 4, [6], [3]), (1, 144, 4, [3, 1], [3, 1]),
+                                      # rows beyond 64 tokens: the bfloat16 mode runs them in chunks of 64 side by side
+                                      (2, 64, 8, [1, 64, 65, 300, 128], [5, 4, 3, 2, 1]), (3, 24, 4, [129, 2], [1, 2]), (1, 80, 4, [70], [2])):
         step = FakeStep(lens, slots)
         T, n = step.num_tokens, H * d
         cols = dict(r=2, k=2 + n, v=3 + 2 * n, g=3 + 3 * n, a=4 + 4 * n, w=4 + 5 * n)
