@@ -55,7 +55,11 @@ qkv_finish_kernel(FinishArgs a) {
     for (int i = threadIdx.x; i < nk; i += blockDim.x) ss = fmaf(k[i], k[i], ss);
     rk = 1.0f / sqrtf(block_sum(ss, scratch) / (float)nk + a.eps);
   }
+  // the angles' cosines and sines once a token: every head turns by the same ones
+  extern __shared__ float cs[];                 // cos [nf], sin [nf]
   const float pos = (float)a.positions[t];
+  for (int i = threadIdx.x; i < a.nf; i += blockDim.x) sincosf(pos * a.inv_freq[i], &cs[a.nf + i], &cs[i]);
+  __syncthreads();
   const int turned = 2 * a.nf;
   auto value = [&](const float* x, const float* w, float r, int h, int d) -> float {
     auto normed = [&](int e) { return w ? x[h * a.dim + e] * r * w[h * a.dim + e] : x[h * a.dim + e]; };
@@ -65,8 +69,7 @@ qkv_finish_kernel(FinishArgs a) {
     bool first;
     pair_of(d, a.nf, a.layout, i, partner, first);
     const float other = normed(partner);
-    float s, c;
-    sincosf(pos * a.inv_freq[i], &s, &c);
+    const float c = cs[i], s = cs[a.nf + i];
     float o1, o2;
     if (first) {
       rotate_pair(own, other, c, s, o1, o2);
@@ -114,8 +117,9 @@ MIE_EXPORT int mie_qkv_finish(const float* sums, long ld, int q_col, int k_col, 
   if (v_col < 0 && vdim != dim) MIE_FAIL("qkv_finish: values that are the keys have their size");
   FinishArgs a{sums, ld, q_col, k_col, v_col, q_norm, k_norm, eps, inv_freq, nf, layout, q_head_scale, positions, slots,
                q_out, k_cache, v_cache, Hq, Hkv, dim, vdim, P, page};
-  if (dtype == MIE_F32) hipLaunchKernelGGL(qkv_finish_kernel<float>, dim3(tokens), dim3(256), 0, s, a);
-  else if (dtype == MIE_BF16) hipLaunchKernelGGL(qkv_finish_kernel<bf16>, dim3(tokens), dim3(256), 0, s, a);
+  const size_t lds = (size_t)2 * (nf > 0 ? nf : 1) * sizeof(float);
+  if (dtype == MIE_F32) hipLaunchKernelGGL(qkv_finish_kernel<float>, dim3(tokens), dim3(256), lds, s, a);
+  else if (dtype == MIE_BF16) hipLaunchKernelGGL(qkv_finish_kernel<bf16>, dim3(tokens), dim3(256), lds, s, a);
   else MIE_FAIL("qkv_finish: dtype code %d", dtype);
   MIE_CHECK_LAUNCH("qkv_finish");
   return 0;

@@ -22,29 +22,37 @@ __global__ void __launch_bounds__(256)
 delta_prepare_kernel(const float* __restrict__ sums, long ld, int k_col, int a_col, int w_col, const float* __restrict__ w_decay,
                      int rank, const float* __restrict__ decay_bias, float decay_scale, const float* __restrict__ removal_bias,
                      float* __restrict__ prep, int H, int d) {
-  extern __shared__ float lds[];          // inner [rank], head sums [H]
-  float* inner = lds;
-  float* ss = lds + rank;
+  extern __shared__ __align__(16) float inner[];          // [rank], the decay's inner activations after their tanh
   const int t = blockIdx.x, n = H * d;
   const float* row = sums + (size_t)t * ld;
   for (int j = threadIdx.x; j < rank; j += blockDim.x) inner[j] = tanhf(row[w_col + j]);
-  for (int h = threadIdx.x; h < H; h += blockDim.x) {
-    float s = 0.f;
-    for (int i = 0; i < d; ++i) s = fmaf(row[k_col + h * d + i], row[k_col + h * d + i], s);
-    ss[h] = s;
-  }
   __syncthreads();
-  float* out = prep + (size_t)t * 3 * n;
-  for (int c = threadIdx.x; c < n; c += blockDim.x) {
-    float z = decay_bias[c];
-    const float* w = w_decay + (size_t)c * rank;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;    // a thread a channel, 256 channels a workgroup
+  if (c >= n) return;
+  // the head's sum of squares, by every thread of the head in the same order
+  const float* kh = row + k_col + (c / d) * d;
+  float ss = 0.f;
+  for (int i = 0; i < d; ++i) ss = fmaf(kh[i], kh[i], ss);
+  float z = decay_bias[c];
+  const float* w = w_decay + (size_t)c * rank;
+  if ((rank & 3) == 0 && (((uintptr_t)w_decay) & 15) == 0) {
+    for (int j = 0; j < rank; j += 4) {
+      const float4 wv = *reinterpret_cast<const float4*>(w + j);
+      const float4 iv = *reinterpret_cast<const float4*>(inner + j);
+      z = fmaf(wv.x, iv.x, z);
+      z = fmaf(wv.y, iv.y, z);
+      z = fmaf(wv.z, iv.z, z);
+      z = fmaf(wv.w, iv.w, z);
+    }
+  } else {
     for (int j = 0; j < rank; ++j) z = fmaf(w[j], inner[j], z);
-    const float a = mie_sigmoid(row[a_col + c] + removal_bias[c]);
-    const float u = row[k_col + c] / sqrtf(ss[c / d] + 1e-6f);
-    out[c] = expf(-decay_scale * mie_sigmoid(z));
-    out[n + c] = a * u;
-    out[2 * n + c] = u;
   }
+  const float a = mie_sigmoid(row[a_col + c] + removal_bias[c]);
+  const float u = row[k_col + c] / sqrtf(ss + 1e-6f);
+  float* out = prep + (size_t)t * 3 * n;
+  out[c] = expf(-decay_scale * mie_sigmoid(z));
+  out[n + c] = a * u;
+  out[2 * n + c] = u;
 }
 
 enum { SCAN_WHOLE = 0, SCAN_SUMMARY = 1, SCAN_FROM_START = 2 };
@@ -248,9 +256,10 @@ MIE_EXPORT int mie_delta_rule(const float* sums, long ld, int r_col, int k_col, 
   if (H > 65535) MIE_FAIL("delta_rule: %d heads is beyond the grid", H);
   if (chunk_tokens < 0 || (chunk_tokens > 0 && (max_chunks < 1 || !summaries || !starts)))
     MIE_FAIL("delta_rule: chunks of %d tokens, %d a row, need their scratch", chunk_tokens, max_chunks);
-  const size_t lds = (size_t)(rank + H) * sizeof(float);
-  if (lds > 60 * 1024) MIE_FAIL("delta_rule: inner size %d and %d heads do not fit the LDS", rank, H);
-  hipLaunchKernelGGL(delta_prepare_kernel, dim3(tokens), dim3(256), lds, s, sums, ld, k_col, a_col, w_col, w_decay, rank,
+  const size_t lds = (size_t)(rank + 4) * sizeof(float);
+  if (lds > 60 * 1024) MIE_FAIL("delta_rule: an inner size of %d does not fit the LDS", rank);
+  if ((H * d + 255) / 256 > 65535) MIE_FAIL("delta_rule: %d channels is beyond the grid", H * d);
+  hipLaunchKernelGGL(delta_prepare_kernel, dim3(tokens, (H * d + 255) / 256), dim3(256), lds, s, sums, ld, k_col, a_col, w_col, w_decay, rank,
                      decay_bias, decay_scale, removal_bias, prep, H, d);
   MIE_CHECK_LAUNCH("delta_rule (prepare)");
   ScanArgs a{sums, ld, r_col, k_col, v_col, g_col, prep, norm_weight, eps, state, row_start, slots, out, summaries, starts,

@@ -340,6 +340,49 @@ MIE_EXPORT int mie_rmsnorm_columns(const float* x, long ldx, const void* weight,
 
 // ---- stream[row] += scale * (a * rstd(a) * wa + b * rstd(b) * wb): two branch outputs, each normed over the row, joined
 // and added in one pass (b null: one).  One workgroup a row, float32 throughout.
+// widths that are a multiple of 4 up to 8192: 16-byte loads, both rows read once and kept in registers
+constexpr int NSA_V = 8;
+__global__ void __launch_bounds__(NORM_THREADS)
+normed_sum_add_vec_kernel(float* __restrict__ stream, const float* __restrict__ a, const float* __restrict__ wa,
+                          const float* __restrict__ b, const float* __restrict__ wb, int width, float eps, float scale) {
+  __shared__ float scratch[16];
+  const size_t base = (size_t)blockIdx.x * width;
+  const int nv = width / 4;
+  float4 va[NSA_V], vb[NSA_V];
+  float sa = 0.f, sb = 0.f;
+#pragma unroll
+  for (int k = 0; k < NSA_V; ++k) {
+    const int i = threadIdx.x + k * NORM_THREADS;
+    va[k] = i < nv ? reinterpret_cast<const float4*>(a + base)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    vb[k] = (b && i < nv) ? reinterpret_cast<const float4*>(b + base)[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    sa = fmaf(va[k].x, va[k].x, fmaf(va[k].y, va[k].y, fmaf(va[k].z, va[k].z, fmaf(va[k].w, va[k].w, sa))));
+    sb = fmaf(vb[k].x, vb[k].x, fmaf(vb[k].y, vb[k].y, fmaf(vb[k].z, vb[k].z, fmaf(vb[k].w, vb[k].w, sb))));
+  }
+  const float ra = 1.0f / sqrtf(block_sum(sa, scratch) / (float)width + eps);
+  const float rb = b ? 1.0f / sqrtf(block_sum(sb, scratch) / (float)width + eps) : 0.f;
+#pragma unroll
+  for (int k = 0; k < NSA_V; ++k) {
+    const int i = threadIdx.x + k * NORM_THREADS;
+    if (i < nv) {
+      const float4 ga = reinterpret_cast<const float4*>(wa)[i];
+      float4 v = make_float4(va[k].x * ra * ga.x, va[k].y * ra * ga.y, va[k].z * ra * ga.z, va[k].w * ra * ga.w);
+      if (b) {
+        const float4 gb = reinterpret_cast<const float4*>(wb)[i];
+        v.x += vb[k].x * rb * gb.x;
+        v.y += vb[k].y * rb * gb.y;
+        v.z += vb[k].z * rb * gb.z;
+        v.w += vb[k].w * rb * gb.w;
+      }
+      float4 st = reinterpret_cast<float4*>(stream + base)[i];
+      st.x += scale * v.x;
+      st.y += scale * v.y;
+      st.z += scale * v.z;
+      st.w += scale * v.w;
+      reinterpret_cast<float4*>(stream + base)[i] = st;
+    }
+  }
+}
+
 __global__ void __launch_bounds__(NORM_THREADS)
 normed_sum_add_kernel(float* __restrict__ stream, const float* __restrict__ a, const float* __restrict__ wa,
                       const float* __restrict__ b, const float* __restrict__ wb, int width, float eps, float scale) {
@@ -363,7 +406,11 @@ MIE_EXPORT int mie_normed_sum_add(float* stream, const float* a, const float* wa
                                   int width, float eps, float scale, hipStream_t s) {
   if (rows <= 0) return 0;
   if (width <= 0 || !stream || !a || !wa || (b && !wb)) MIE_FAIL("normed_sum_add: width %d or a missing operand", width);
-  hipLaunchKernelGGL(normed_sum_add_kernel, dim3(rows), dim3(NORM_THREADS), 0, s, stream, a, wa, b, wb, width, eps, scale);
+  const bool aligned = !(((uintptr_t)stream | (uintptr_t)a | (uintptr_t)wa | (uintptr_t)b | (uintptr_t)wb) & 15);
+  if (width % 4 == 0 && width <= 4 * NSA_V * NORM_THREADS && aligned)
+    hipLaunchKernelGGL(normed_sum_add_vec_kernel, dim3(rows), dim3(NORM_THREADS), 0, s, stream, a, wa, b, wb, width, eps, scale);
+  else
+    hipLaunchKernelGGL(normed_sum_add_kernel, dim3(rows), dim3(NORM_THREADS), 0, s, stream, a, wa, b, wb, width, eps, scale);
   MIE_CHECK_LAUNCH("normed_sum_add");
   return 0;
 }
@@ -418,6 +465,87 @@ norm_pair_conv_kernel(const float* __restrict__ stream, const float* __restrict_
   }
 }
 
+// The same for widths that are a multiple of 4 up to 8192, the number of taps known at compile time: 16-byte loads, the
+// token's own row read once and kept in registers, four channels' taps as K consecutive 16-byte loads.
+constexpr int NPC_V = 8;
+__device__ __forceinline__ void store4(float* p, float a, float b, float c, float d) {
+  *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
+}
+__device__ __forceinline__ void store4(bf16* p, float a, float b, float c, float d) {
+  const bf16 v[4] = {__float2bfloat16(a), __float2bfloat16(b), __float2bfloat16(c), __float2bfloat16(d)};
+  *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(v);
+}
+
+template <typename TO, int K>
+__global__ void __launch_bounds__(NORM_THREADS)
+norm_pair_conv_vec_kernel(const float* __restrict__ stream, const float* __restrict__ w1, const float* __restrict__ w2,
+                          const float* __restrict__ taps, const float* __restrict__ tail, const int* __restrict__ token_row,
+                          const int* __restrict__ row_start, const int* __restrict__ slots, TO* __restrict__ xm,
+                          TO* __restrict__ y, float* __restrict__ rstd_out, int width, float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x, nv = width / 4;
+  const int r = token_row[t], j = t - row_start[r];
+  const int have = j < K - 1 ? j : K - 1;            // rows before this one that are in the step
+  const float4* own = reinterpret_cast<const float4*>(stream + (size_t)t * width);
+  float4 xo[NPC_V];
+  float ss[K];
+#pragma unroll
+  for (int b = 0; b < K; ++b) ss[b] = 0.f;
+#pragma unroll
+  for (int k = 0; k < NPC_V; ++k) {
+    const int i = threadIdx.x + k * NORM_THREADS;
+    xo[k] = i < nv ? own[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    ss[0] = fmaf(xo[k].x, xo[k].x, fmaf(xo[k].y, xo[k].y, fmaf(xo[k].z, xo[k].z, fmaf(xo[k].w, xo[k].w, ss[0]))));
+#pragma unroll
+    for (int b = 1; b < K; ++b)
+      if (b <= have && i < nv) {
+        const float4 v = (own - (size_t)b * nv)[i];
+        ss[b] = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss[b]))));
+      }
+  }
+  float rstd[K];
+#pragma unroll
+  for (int b = 0; b < K; ++b)
+    rstd[b] = b <= have ? 1.0f / sqrtf(block_sum(ss[b], scratch) / (float)width + eps) : 0.f;    // ``have`` is the workgroup's
+  if (threadIdx.x == 0) rstd_out[t] = rstd[0];
+  const float4* tl = reinterpret_cast<const float4*>(tail + (size_t)slots[r] * (K > 1 ? K - 1 : 1) * width);
+#pragma unroll
+  for (int k = 0; k < NPC_V; ++k) {
+    const int i = threadIdx.x + k * NORM_THREADS;
+    if (i >= nv) continue;
+    const float4 g = reinterpret_cast<const float4*>(w1)[i];
+    float tp[4 * K];                                  // taps of channels 4 i .. 4 i + 3, K each
+#pragma unroll
+    for (int q = 0; q < K; ++q) {
+      const float4 v = reinterpret_cast<const float4*>(taps + (size_t)i * 4 * K)[q];
+      tp[4 * q] = v.x, tp[4 * q + 1] = v.y, tp[4 * q + 2] = v.z, tp[4 * q + 3] = v.w;
+    }
+    const float h0[4] = {xo[k].x * rstd[0] * g.x, xo[k].y * rstd[0] * g.y, xo[k].z * rstd[0] * g.z, xo[k].w * rstd[0] * g.w};
+    float acc[4] = {h0[0], h0[1], h0[2], h0[3]};
+#pragma unroll
+    for (int b = 0; b < K; ++b) {
+      float h[4];
+      if (b == 0) {
+        h[0] = h0[0], h[1] = h0[1], h[2] = h0[2], h[3] = h0[3];
+      } else if (b <= have) {
+        const float4 v = (own - (size_t)b * nv)[i];
+        h[0] = v.x * rstd[b] * g.x, h[1] = v.y * rstd[b] * g.y, h[2] = v.z * rstd[b] * g.z, h[3] = v.w * rstd[b] * g.w;
+      } else {
+        const float4 v = tl[(size_t)(K - 1 + j - b) * nv + i];
+        h[0] = v.x, h[1] = v.y, h[2] = v.z, h[3] = v.w;
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] = fmaf(tp[e * K + (K - 1 - b)], h[e], acc[e]);
+    }
+    store4(xm + (size_t)t * width + 4 * i, acc[0], acc[1], acc[2], acc[3]);
+    if (w2) {
+      const float4 g2 = reinterpret_cast<const float4*>(w2)[i];
+      store4(y + (size_t)t * width + 4 * i, xo[k].x * rstd[0] * g2.x, xo[k].y * rstd[0] * g2.y, xo[k].z * rstd[0] * g2.z,
+             xo[k].w * rstd[0] * g2.w);
+    }
+  }
+}
+
 __global__ void __launch_bounds__(256)
 norm_conv_tail_kernel(const float* __restrict__ stream, const float* __restrict__ w1, const float* __restrict__ rstd,
                       float* __restrict__ tail, const int* __restrict__ row_start, const int* __restrict__ slots, int width,
@@ -441,13 +569,28 @@ MIE_EXPORT int mie_norm_pair_conv(const float* stream, const float* w1, const fl
   if (tokens <= 0 || rows <= 0) return 0;
   if (width <= 0 || K < 1 || K > CONV_MAX_TAPS) MIE_FAIL("norm_pair_conv: width %d, %d taps (1 to %d)", width, K, CONV_MAX_TAPS);
   if (!stream || !w1 || !taps || !tail || !xm || !rstd || (w2 && !y)) MIE_FAIL("norm_pair_conv: a missing operand");
-  if (out_dtype == MIE_F32)
+  if (out_dtype != MIE_F32 && out_dtype != MIE_BF16) MIE_FAIL("norm_pair_conv: out dtype code %d", out_dtype);
+  const bool aligned = !(((uintptr_t)stream | (uintptr_t)w1 | (uintptr_t)w2 | (uintptr_t)taps | (uintptr_t)tail | (uintptr_t)xm |
+                          (uintptr_t)y) & 15);
+  if (width % 4 == 0 && width <= 4 * NPC_V * NORM_THREADS && aligned) {
+#define NPC_LAUNCH(TO_, K_)                                                                                                   \
+  hipLaunchKernelGGL((norm_pair_conv_vec_kernel<TO_, K_>), dim3(tokens), dim3(NORM_THREADS), 0, s, stream, w1, w2, taps, tail, \
+                     token_row, row_start, slots, (TO_*)xm, (TO_*)y, rstd, width, eps)
+#define NPC_TAPS(TO_)                                                                                           \
+  switch (K) {                                                                                                  \
+    case 1: NPC_LAUNCH(TO_, 1); break; case 2: NPC_LAUNCH(TO_, 2); break; case 3: NPC_LAUNCH(TO_, 3); break;     \
+    case 4: NPC_LAUNCH(TO_, 4); break; case 5: NPC_LAUNCH(TO_, 5); break; case 6: NPC_LAUNCH(TO_, 6); break;     \
+    case 7: NPC_LAUNCH(TO_, 7); break; default: NPC_LAUNCH(TO_, 8); break;                                       \
+  }
+    if (out_dtype == MIE_F32) { NPC_TAPS(float) } else { NPC_TAPS(bf16) }
+#undef NPC_TAPS
+#undef NPC_LAUNCH
+  } else if (out_dtype == MIE_F32)
     hipLaunchKernelGGL(norm_pair_conv_kernel<float>, dim3(tokens), dim3(NORM_THREADS), 0, s, stream, w1, w2, taps, tail, token_row,
                        row_start, slots, (float*)xm, (float*)y, rstd, width, K, eps);
-  else if (out_dtype == MIE_BF16)
+  else
     hipLaunchKernelGGL(norm_pair_conv_kernel<bf16>, dim3(tokens), dim3(NORM_THREADS), 0, s, stream, w1, w2, taps, tail, token_row,
                        row_start, slots, (bf16*)xm, (bf16*)y, rstd, width, K, eps);
-  else MIE_FAIL("norm_pair_conv: out dtype code %d", out_dtype);
   MIE_CHECK_LAUNCH("norm_pair_conv");
   if (K > 1) {
     hipLaunchKernelGGL(norm_conv_tail_kernel, dim3(rows, (width + 255) / 256), dim3(256), 0, s, stream, w1, rstd, tail, row_start,
