@@ -13,46 +13,83 @@
 // Rows run whole (one chunk: S from state[slot], left there afterwards), or, long rows, in chunks of L tokens side by
 // side in three passes, since a chunk acts on the state it starts from as S_end = P S_start + B with P and B of the
 // chunk's own tokens:  (1) every chunk but a row's last computes P (the recurrence without k v^T on the identity) and
-// B (the recurrence on zero);  (2) per row and head, chunk after chunk, S_start(c + 1) = P_c S_start(c) + B_c from
+// B (the recurrence on zero), a thread carrying the same column of both;  (2) per row and head, chunk after chunk, S_start(c + 1) = P_c S_start(c) + B_c from
 // state[slot] (16 columns a workgroup; columns do not mix);  (3) every chunk runs its tokens from its S_start and writes
 // the outputs, a row's last chunk leaves state[slot].  The two ways differ by the rounding of pass 2 alone.
 #include "common.hpp"
 
+constexpr int PT_MAX = 16;       // most tokens a workgroup of delta_prepare takes: a channel's row of the decay matrix is read once for all of them
+
+// RMAX > 0: inner sizes up to RMAX, the channel's row of the matrix in registers; 0: any inner size, the row read from memory
+template <int RMAX>
 __global__ void __launch_bounds__(256)
 delta_prepare_kernel(const float* __restrict__ sums, long ld, int k_col, int a_col, int w_col, const float* __restrict__ w_decay,
                      int rank, const float* __restrict__ decay_bias, float decay_scale, const float* __restrict__ removal_bias,
-                     float* __restrict__ prep, int H, int d) {
-  extern __shared__ __align__(16) float inner[];          // [rank], the decay's inner activations after their tanh
-  const int t = blockIdx.x, n = H * d;
-  const float* row = sums + (size_t)t * ld;
-  for (int j = threadIdx.x; j < rank; j += blockDim.x) inner[j] = tanhf(row[w_col + j]);
-  __syncthreads();
-  const int c = blockIdx.y * blockDim.x + threadIdx.x;    // a thread a channel, 256 channels a workgroup
-  if (c >= n) return;
-  // the head's sum of squares, by every thread of the head in the same order
-  const float* kh = row + k_col + (c / d) * d;
-  float ss = 0.f;
-  for (int i = 0; i < d; ++i) ss = fmaf(kh[i], kh[i], ss);
-  float z = decay_bias[c];
-  const float* w = w_decay + (size_t)c * rank;
-  if ((rank & 3) == 0 && (((uintptr_t)w_decay) & 15) == 0) {
-    for (int j = 0; j < rank; j += 4) {
-      const float4 wv = *reinterpret_cast<const float4*>(w + j);
-      const float4 iv = *reinterpret_cast<const float4*>(inner + j);
-      z = fmaf(wv.x, iv.x, z);
-      z = fmaf(wv.y, iv.y, z);
-      z = fmaf(wv.z, iv.z, z);
-      z = fmaf(wv.w, iv.w, z);
-    }
-  } else {
-    for (int j = 0; j < rank; ++j) z = fmaf(w[j], inner[j], z);
+                     float* __restrict__ prep, int tokens, int H, int d, int heads_here, int PT) {
+  extern __shared__ __align__(16) float prep_lds[];
+  const int rank4 = RMAX > 0 ? RMAX : (rank + 3) & ~3;
+  float* inner = prep_lds;                       // [PT][rank4]: the decay's inner activations after their tanh
+  float* ssq = prep_lds + (size_t)PT * rank4;    // [PT][heads_here]: sum of squares of the keys of the heads this workgroup touches
+  const int t0 = blockIdx.x * PT, n = H * d;
+  const int nt = tokens - t0 < PT ? tokens - t0 : PT;
+  const int c0 = blockIdx.y * 256, h0 = c0 / d;
+  for (int e = threadIdx.x; e < nt * rank4; e += blockDim.x) {
+    const int tt = e / rank4, j = e % rank4;
+    inner[e] = j < rank ? tanhf(sums[(size_t)(t0 + tt) * ld + w_col + j]) : 0.f;
   }
-  const float a = mie_sigmoid(row[a_col + c] + removal_bias[c]);
-  const float u = row[k_col + c] / sqrtf(ss + 1e-6f);
-  float* out = prep + (size_t)t * 3 * n;
-  out[c] = expf(-decay_scale * mie_sigmoid(z));
-  out[n + c] = a * u;
-  out[2 * n + c] = u;
+  for (int e = threadIdx.x; e < nt * heads_here; e += blockDim.x) {
+    const int tt = e / heads_here, h = h0 + e % heads_here;
+    float s = 0.f;
+    if (h < H) {
+      const float* kh = sums + (size_t)(t0 + tt) * ld + k_col + (size_t)h * d;
+      for (int i = 0; i < d; ++i) s = fmaf(kh[i], kh[i], s);      // the same order whatever the step holds
+    }
+    ssq[e] = s;
+  }
+  __syncthreads();
+  const int c = c0 + threadIdx.x;                // a thread a channel
+  if (c >= n) return;
+  const float* w = w_decay + (size_t)c * rank;
+  const float zb = decay_bias[c], rb = removal_bias[c];
+  const int hl = c / d - h0;
+  const bool vec = (rank & 3) == 0 && (((uintptr_t)w_decay) & 15) == 0;
+  float wreg[RMAX > 0 ? RMAX : 1];
+  if (RMAX > 0) {
+#pragma unroll
+    for (int j = 0; j < RMAX; ++j) wreg[j] = j < rank ? w[j] : 0.f;
+  }
+  for (int tt = 0; tt < nt; ++tt) {
+    float z = zb;
+    const float* in = inner + (size_t)tt * rank4;
+    if (RMAX > 0) {
+#pragma unroll
+      for (int j = 0; j < RMAX; j += 4) {          // inner is zero beyond the inner size
+        const float4 iv = *reinterpret_cast<const float4*>(in + j);
+        z = fmaf(wreg[j], iv.x, z);
+        z = fmaf(wreg[j + 1], iv.y, z);
+        z = fmaf(wreg[j + 2], iv.z, z);
+        z = fmaf(wreg[j + 3], iv.w, z);
+      }
+    } else if (vec) {
+      for (int j = 0; j < rank; j += 4) {        // the row of the matrix stays in the cache nearest this thread over the tokens
+        const float4 wv = *reinterpret_cast<const float4*>(w + j);
+        const float4 iv = *reinterpret_cast<const float4*>(in + j);
+        z = fmaf(wv.x, iv.x, z);
+        z = fmaf(wv.y, iv.y, z);
+        z = fmaf(wv.z, iv.z, z);
+        z = fmaf(wv.w, iv.w, z);
+      }
+    } else {
+      for (int j = 0; j < rank; ++j) z = fmaf(w[j], in[j], z);
+    }
+    const float* row = sums + (size_t)(t0 + tt) * ld;
+    const float a = mie_sigmoid(row[a_col + c] + rb);
+    const float u = row[k_col + c] / sqrtf(ssq[tt * heads_here + hl] + 1e-6f);
+    float* out = prep + (size_t)(t0 + tt) * 3 * n;
+    out[c] = expf(-decay_scale * mie_sigmoid(z));
+    out[n + c] = a * u;
+    out[2 * n + c] = u;
+  }
 }
 
 enum { SCAN_WHOLE = 0, SCAN_SUMMARY = 1, SCAN_FROM_START = 2 };
@@ -68,7 +105,7 @@ struct ScanArgs {
   int H, d, L, max_chunks, mode;
 };
 
-template <int DMAX, typename TO>
+template <int DMAX, typename TO, bool SUMMARY>
 __global__ void __launch_bounds__(DMAX < 64 ? 64 : DMAX)
 delta_scan_kernel(ScanArgs a) {
   constexpr int NT = DMAX < 64 ? 64 : DMAX;
@@ -81,16 +118,19 @@ delta_scan_kernel(ScanArgs a) {
   if (t0 >= row_end) return;                                   // the whole workgroup: this row has no such chunk
   const int t1 = t0 + a.L < row_end ? t0 + a.L : row_end;
   const bool last = t1 == row_end;
-  const bool summary = a.mode == SCAN_SUMMARY, identity = summary && blockIdx.z == 1;
+  constexpr bool summary = SUMMARY;                            // one thread carries column j of B (in S) and of P (in Q)
   if (summary && last) return;                                 // nobody starts from the end of a row's last chunk
   const bool live = j < d;
   const int jj = live ? j : 0;
   float* sp = a.state + ((size_t)a.slots[row] * a.H + h) * d * d;
   const size_t ch = (size_t)blockIdx.x * a.H + h;
   float S[DMAX];
+  float Q[SUMMARY ? DMAX : 1];
   if (summary) {
 #pragma unroll
-    for (int i = 0; i < DMAX; ++i) S[i] = identity && i == jj ? 1.f : 0.f;
+    for (int i = 0; i < DMAX; ++i) S[i] = 0.f;
+#pragma unroll
+    for (int i = 0; i < (SUMMARY ? DMAX : 1); ++i) Q[i] = live && i == j ? 1.f : 0.f;
   } else {
     const float* from = a.mode == SCAN_FROM_START ? a.starts + ch * d * d : sp;
 #pragma unroll
@@ -138,21 +178,30 @@ delta_scan_kernel(ScanArgs a) {
       const float* u = stage[tt][2] + lane0;
       const float* k = stage[tt][3] + lane0;
       const float* r = stage[tt][4] + lane0;
-      const float v = identity ? 0.f : stage[tt][5][jj];
-      float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+      const float v = stage[tt][5][jj];
+      float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f, q0 = 0.f, q1 = 0.f, q2 = 0.f, q3 = 0.f;
 #pragma unroll
       for (int i = 0; i < DMAX; i += 4) {
         s0 = fmaf(u[i], S[i], s0);
         s1 = fmaf(u[i + 1], S[i + 1], s1);
         s2 = fmaf(u[i + 2], S[i + 2], s2);
         s3 = fmaf(u[i + 3], S[i + 3], s3);
+        if (summary) {
+          q0 = fmaf(u[i], Q[i], q0);
+          q1 = fmaf(u[i + 1], Q[i + 1], q1);
+          q2 = fmaf(u[i + 2], Q[i + 2], q2);
+          q3 = fmaf(u[i + 3], Q[i + 3], q3);
+        }
       }
-      const float seen = (s0 + s1) + (s2 + s3);
+      const float seen = (s0 + s1) + (s2 + s3), seen_q = (q0 + q1) + (q2 + q3);
       float o0 = 0.f, o1 = 0.f, o2 = 0.f, o3 = 0.f;
 #pragma unroll
       for (int i = 0; i < DMAX; i += 4) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) S[i + e] = fmaf(k[i + e], v, fmaf(-au[i + e], seen, decay[i + e] * S[i + e]));
+        for (int e = 0; e < 4; ++e) {
+          S[i + e] = fmaf(k[i + e], v, fmaf(-au[i + e], seen, decay[i + e] * S[i + e]));
+          if (summary) Q[i + e] = fmaf(-au[i + e], seen_q, decay[i + e] * Q[i + e]);       // no k v^T: what the start state becomes
+        }
         if (!summary) {
           o0 = fmaf(S[i], r[i], o0);
           o1 = fmaf(S[i + 1], r[i + 1], o1);
@@ -172,11 +221,16 @@ delta_scan_kernel(ScanArgs a) {
     }
   }
   if (!live) return;
-  float* to = summary ? a.summaries + (ch * 2 + blockIdx.z) * d * d : sp;
+  float* to = summary ? a.summaries + ch * 2 * d * d : sp;
   if (summary || last) {
 #pragma unroll
     for (int i = 0; i < DMAX; ++i)
       if (i < d) to[(size_t)i * d + j] = S[i];
+  }
+  if (summary) {
+#pragma unroll
+    for (int i = 0; i < (SUMMARY ? DMAX : 1); ++i)
+      if (i < d) to[(size_t)(d + i) * d + j] = Q[i];
   }
 }
 
@@ -197,6 +251,18 @@ delta_fold_kernel(const float* __restrict__ summaries, float* __restrict__ start
     col[e] = j0 + jl < d ? sp[(size_t)i * d + j0 + jl] : 0.f;
   }
   __syncthreads();
+  // P of a chunk comes in through registers while the chunk before is folded (d * d / 256 numbers a thread)
+  const int per = (d * d + 255) / 256;
+  float pre[16];                                 // the first 16 of them; the rest, for d > 64, is read when needed
+  auto ask = [&](int c) {
+    const float* P = summaries + ((((size_t)row * max_chunks + c) * H + h) * 2 + 1) * d * d;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const int e = threadIdx.x + k * 256;
+      pre[k] = (k < per && e < d * d) ? P[e] : 0.f;
+    }
+  };
+  if (chunks > 1) ask(0);
   for (int c = 0; c < chunks; ++c) {
     const size_t ch = ((size_t)row * max_chunks + c) * H + h;
     float* st = starts + ch * d * d;
@@ -205,8 +271,14 @@ delta_fold_kernel(const float* __restrict__ summaries, float* __restrict__ start
     if (c + 1 == chunks) break;
     const float* B = summaries + ch * 2 * d * d;
     const float* P = B + (size_t)d * d;
-    for (int e = threadIdx.x; e < d * d; e += blockDim.x) pm[(e / d) * (d + 1) + e % d] = P[e];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      const int e = threadIdx.x + k * 256;
+      if (k < per && e < d * d) pm[(e / d) * (d + 1) + e % d] = pre[k];
+    }
+    for (int e = threadIdx.x + 16 * 256; e < d * d; e += blockDim.x) pm[(e / d) * (d + 1) + e % d] = P[e];
     __syncthreads();
+    if (c + 2 < chunks) ask(c + 1);
     // every thread's new values first (up to four quads of columns at d = 256), then all of them into the LDS
     float4 fresh[4];
 #pragma unroll
@@ -256,34 +328,43 @@ MIE_EXPORT int mie_delta_rule(const float* sums, long ld, int r_col, int k_col, 
   if (H > 65535) MIE_FAIL("delta_rule: %d heads is beyond the grid", H);
   if (chunk_tokens < 0 || (chunk_tokens > 0 && (max_chunks < 1 || !summaries || !starts)))
     MIE_FAIL("delta_rule: chunks of %d tokens, %d a row, need their scratch", chunk_tokens, max_chunks);
-  const size_t lds = (size_t)(rank + 4) * sizeof(float);
+  const int heads_here = 255 / d + 2;           // heads a workgroup's 256 channels can touch
+  // few tokens: a workgroup a token; many: up to PT_MAX tokens a workgroup, the matrix read once for them
+  const int pt = tokens <= 64 ? 1 : tokens < 64 * PT_MAX ? (tokens + 63) / 64 : PT_MAX;
+  const int rmax = rank <= 16 ? 16 : rank <= 64 ? 64 : 0;
+  const size_t lds = ((size_t)pt * (rmax ? rmax : (rank + 3) & ~3) + (size_t)pt * heads_here) * sizeof(float);
   if (lds > 60 * 1024) MIE_FAIL("delta_rule: an inner size of %d does not fit the LDS", rank);
   if ((H * d + 255) / 256 > 65535) MIE_FAIL("delta_rule: %d channels is beyond the grid", H * d);
-  hipLaunchKernelGGL(delta_prepare_kernel, dim3(tokens, (H * d + 255) / 256), dim3(256), lds, s, sums, ld, k_col, a_col, w_col, w_decay, rank,
-                     decay_bias, decay_scale, removal_bias, prep, H, d);
+#define DP_LAUNCH(RMAX_)                                                                                                     \
+  hipLaunchKernelGGL(delta_prepare_kernel<RMAX_>, dim3((tokens + pt - 1) / pt, (H * d + 255) / 256), dim3(256), lds, s, sums, ld, \
+                     k_col, a_col, w_col, w_decay, rank, decay_bias, decay_scale, removal_bias, prep, tokens, H, d, heads_here, pt)
+  if (rmax == 16) DP_LAUNCH(16);
+  else if (rmax == 64) DP_LAUNCH(64);
+  else DP_LAUNCH(0);
+#undef DP_LAUNCH
   MIE_CHECK_LAUNCH("delta_rule (prepare)");
   ScanArgs a{sums, ld, r_col, k_col, v_col, g_col, prep, norm_weight, eps, state, row_start, slots, out, summaries, starts,
              H, d, chunk_tokens > 0 ? chunk_tokens : 1 << 30, chunk_tokens > 0 ? max_chunks : 1, SCAN_WHOLE};
-#define DR_LAUNCH(DMAX_, TO_, GRID_) \
-  hipLaunchKernelGGL((delta_scan_kernel<DMAX_, TO_>), GRID_, dim3(DMAX_ < 64 ? 64 : DMAX_), 0, s, a)
-#define DR_SIZES(TO_, GRID_)                      \
-  if (d <= 16) DR_LAUNCH(16, TO_, GRID_);         \
-  else if (d <= 32) DR_LAUNCH(32, TO_, GRID_);    \
-  else if (d <= 64) DR_LAUNCH(64, TO_, GRID_);    \
-  else if (d <= 128) DR_LAUNCH(128, TO_, GRID_);  \
-  else DR_LAUNCH(256, TO_, GRID_)
-#define DR_DTYPES(GRID_)                                   \
-  if (out_dtype == MIE_F32) { DR_SIZES(float, GRID_); }    \
-  else if (out_dtype == MIE_BF16) { DR_SIZES(bf16, GRID_); } \
+#define DR_LAUNCH(DMAX_, TO_, GRID_, SUM_) \
+  hipLaunchKernelGGL((delta_scan_kernel<DMAX_, TO_, SUM_>), GRID_, dim3(DMAX_ < 64 ? 64 : DMAX_), 0, s, a)
+#define DR_SIZES(TO_, GRID_, SUM_)                      \
+  if (d <= 16) DR_LAUNCH(16, TO_, GRID_, SUM_);         \
+  else if (d <= 32) DR_LAUNCH(32, TO_, GRID_, SUM_);    \
+  else if (d <= 64) DR_LAUNCH(64, TO_, GRID_, SUM_);    \
+  else if (d <= 128) DR_LAUNCH(128, TO_, GRID_, SUM_);  \
+  else DR_LAUNCH(256, TO_, GRID_, SUM_)
+#define DR_DTYPES(GRID_, SUM_)                                   \
+  if (out_dtype == MIE_F32) { DR_SIZES(float, GRID_, SUM_); }    \
+  else if (out_dtype == MIE_BF16) { DR_SIZES(bf16, GRID_, SUM_); } \
   else MIE_FAIL("delta_rule: out dtype code %d", out_dtype)
   if (chunk_tokens == 0) {
-    DR_DTYPES(dim3(rows, H));
+    DR_DTYPES(dim3(rows, H), false);
     MIE_CHECK_LAUNCH("delta_rule (scan)");
     return 0;
   }
   if ((long)rows * max_chunks > 2147483647L) MIE_FAIL("delta_rule: %d rows of %d chunks is beyond the grid", rows, max_chunks);
   a.mode = SCAN_SUMMARY;
-  DR_DTYPES(dim3(rows * max_chunks, H, 2));
+  DR_SIZES(float, dim3(rows * max_chunks, H), true);              // writes no outputs: one instantiation serves both dtypes
   MIE_CHECK_LAUNCH("delta_rule (chunk summaries)");
   const size_t fold_lds = ((size_t)d * 16 + (size_t)d * (d + 1)) * sizeof(float);
   if (fold_lds > 64 * 1024) {
@@ -298,7 +379,7 @@ MIE_EXPORT int mie_delta_rule(const float* sums, long ld, int r_col, int k_col, 
                      starts, state, row_start, slots, H, d, chunk_tokens, max_chunks);
   MIE_CHECK_LAUNCH("delta_rule (fold)");
   a.mode = SCAN_FROM_START;
-  DR_DTYPES(dim3(rows * max_chunks, H));
+  DR_DTYPES(dim3(rows * max_chunks, H), false);
   MIE_CHECK_LAUNCH("delta_rule (chunks)");
   return 0;
 #undef DR_DTYPES
