@@ -39,10 +39,11 @@ template <typename TO>
 __global__ void __launch_bounds__(256)
 qkv_finish_kernel(FinishArgs a) {
   __shared__ float scratch[16];
-  const int t = blockIdx.x;
-  const float* row = a.sums + (size_t)t * a.ld;
-  const float* q = row + a.q_col;
-  const float* k = row + a.k_col;
+  // blockIdx.y: which share of the token's numbers this workgroup makes (every one takes the norms' sums itself)
+  const int t = blockIdx.x, first = blockIdx.y * blockDim.x + threadIdx.x, stride = gridDim.y * blockDim.x;
+  const float* __restrict__ row = a.sums + (size_t)t * a.ld;
+  const float* __restrict__ q = row + a.q_col;
+  const float* __restrict__ k = row + a.k_col;
   const int nq = a.Hq * a.dim, nk = a.Hkv * a.dim;
   float rq = 1.f, rk = 1.f;
   if (a.q_norm) {
@@ -78,8 +79,8 @@ qkv_finish_kernel(FinishArgs a) {
     rotate_pair(other, own, c, s, o1, o2);
     return o2;
   };
-  TO* qo = (TO*)a.q_out + (size_t)t * a.Hq * a.P;
-  for (int e = threadIdx.x; e < a.Hq * a.P; e += blockDim.x) {
+  TO* __restrict__ qo = (TO*)a.q_out + (size_t)t * a.Hq * a.P;
+  for (int e = first; e < a.Hq * a.P; e += stride) {
     const int h = e / a.P, d = e - h * a.P;
     float v = 0.f;
     if (d < a.dim) {
@@ -90,10 +91,10 @@ qkv_finish_kernel(FinishArgs a) {
   }
   const int slot = a.slots[t];
   const size_t pg = slot / a.page, off = slot % a.page;
-  TO* kc = (TO*)a.k_cache;
-  TO* vc = (TO*)a.v_cache;
-  const float* vals = a.v_col < 0 ? k : row + a.v_col;
-  for (int e = threadIdx.x; e < a.Hkv * a.P; e += blockDim.x) {
+  TO* __restrict__ kc = (TO*)a.k_cache;
+  TO* __restrict__ vc = (TO*)a.v_cache;
+  const float* __restrict__ vals = a.v_col < 0 ? k : row + a.v_col;
+  for (int e = first; e < a.Hkv * a.P; e += stride) {
     const int g = e / a.P, d = e - g * a.P;
     const float kv = d < a.dim ? value(k, a.k_norm, rk, g, d) : 0.f;
     kc[((pg * a.Hkv + g) * a.page + off) * a.P + d] = from_float<TO>(kv);
@@ -118,8 +119,12 @@ MIE_EXPORT int mie_qkv_finish(const float* sums, long ld, int q_col, int k_col, 
   FinishArgs a{sums, ld, q_col, k_col, v_col, q_norm, k_norm, eps, inv_freq, nf, layout, q_head_scale, positions, slots,
                q_out, k_cache, v_cache, Hq, Hkv, dim, vdim, P, page};
   const size_t lds = (size_t)2 * (nf > 0 ? nf : 1) * sizeof(float);
-  if (dtype == MIE_F32) hipLaunchKernelGGL(qkv_finish_kernel<float>, dim3(tokens), dim3(256), lds, s, a);
-  else if (dtype == MIE_BF16) hipLaunchKernelGGL(qkv_finish_kernel<bf16>, dim3(tokens), dim3(256), lds, s, a);
+  // few tokens: several workgroups a token, so that a decode step's few rows are spread over the GPU
+  const long numbers = (long)(Hq + Hkv) * P;
+  int parts = tokens >= 256 ? 1 : (int)((numbers + 511) / 512);
+  parts = parts < 1 ? 1 : parts > 8 ? 8 : parts;
+  if (dtype == MIE_F32) hipLaunchKernelGGL(qkv_finish_kernel<float>, dim3(tokens, parts), dim3(256), lds, s, a);
+  else if (dtype == MIE_BF16) hipLaunchKernelGGL(qkv_finish_kernel<bf16>, dim3(tokens, parts), dim3(256), lds, s, a);
   else MIE_FAIL("qkv_finish: dtype code %d", dtype);
   MIE_CHECK_LAUNCH("qkv_finish");
   return 0;

@@ -42,7 +42,18 @@ delta_prepare_kernel(const float* __restrict__ sums, long ld, int k_col, int a_c
     float s = 0.f;
     if (h < H) {
       const float* kh = sums + (size_t)(t0 + tt) * ld + k_col + (size_t)h * d;
-      for (int i = 0; i < d; ++i) s = fmaf(kh[i], kh[i], s);      // the same order whatever the step holds
+      if ((d & 3) == 0 && (((uintptr_t)kh) & 15) == 0) {          // the same order whatever the step holds, either way
+#pragma unroll 4
+        for (int i = 0; i < d; i += 4) {
+          const float4 v = *reinterpret_cast<const float4*>(kh + i);
+          s = fmaf(v.x, v.x, s);
+          s = fmaf(v.y, v.y, s);
+          s = fmaf(v.z, v.z, s);
+          s = fmaf(v.w, v.w, s);
+        }
+      } else {
+        for (int i = 0; i < d; ++i) s = fmaf(kh[i], kh[i], s);
+      }
     }
     ssq[e] = s;
   }
