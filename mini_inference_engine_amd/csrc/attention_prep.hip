@@ -11,20 +11,6 @@
 
 enum { LAYOUT_INTERLEAVED = 0, LAYOUT_HALF = 1 };
 
-// element d of a head whose first 2 * nf numbers turn: the pair's angle index, the partner's place, and whether d
-// is the pair's first member
-__device__ __forceinline__ void pair_of(int d, int nf, int layout, int& i, int& partner, bool& first) {
-  if (layout == LAYOUT_INTERLEAVED) {
-    i = d >> 1;
-    partner = d ^ 1;
-    first = (d & 1) == 0;
-  } else {
-    first = d < nf;
-    i = first ? d : d - nf;
-    partner = first ? d + nf : d - nf;
-  }
-}
-
 struct FinishArgs {
   const float* sums; long ld; int q_col, k_col, v_col;      // v_col < 0: the values are the keys as projected
   const float* q_norm; const float* k_norm; float eps;
@@ -39,8 +25,8 @@ template <typename TO>
 __global__ void __launch_bounds__(256)
 qkv_finish_kernel(FinishArgs a) {
   __shared__ float scratch[16];
-  // blockIdx.y: which share of the token's numbers this workgroup makes (every one takes the norms' sums itself)
-  const int t = blockIdx.x, first = blockIdx.y * blockDim.x + threadIdx.x, stride = gridDim.y * blockDim.x;
+  // blockIdx.y: which share of the token's heads this workgroup makes (every one takes the norms' sums itself)
+  const int t = blockIdx.x;
   const float* __restrict__ row = a.sums + (size_t)t * a.ld;
   const float* __restrict__ q = row + a.q_col;
   const float* __restrict__ k = row + a.k_col;
@@ -61,45 +47,42 @@ qkv_finish_kernel(FinishArgs a) {
   const float pos = (float)a.positions[t];
   for (int i = threadIdx.x; i < a.nf; i += blockDim.x) sincosf(pos * a.inv_freq[i], &cs[a.nf + i], &cs[i]);
   __syncthreads();
-  const int turned = 2 * a.nf;
-  auto value = [&](const float* x, const float* w, float r, int h, int d) -> float {
-    auto normed = [&](int e) { return w ? x[h * a.dim + e] * r * w[h * a.dim + e] : x[h * a.dim + e]; };
-    const float own = normed(d);
-    if (d >= turned) return own;
-    int i, partner;
-    bool first;
-    pair_of(d, a.nf, a.layout, i, partner, first);
-    const float other = normed(partner);
-    const float c = cs[i], s = cs[a.nf + i];
-    float o1, o2;
-    if (first) {
-      rotate_pair(own, other, c, s, o1, o2);
-      return o1;
-    }
-    rotate_pair(other, own, c, s, o1, o2);
-    return o2;
-  };
-  TO* __restrict__ qo = (TO*)a.q_out + (size_t)t * a.Hq * a.P;
-  for (int e = first; e < a.Hq * a.P; e += stride) {
-    const int h = e / a.P, d = e - h * a.P;
-    float v = 0.f;
-    if (d < a.dim) {
-      v = value(q, a.q_norm, rq, h, d);
-      if (a.q_head_scale) v *= a.q_head_scale[h];
-    }
-    qo[e] = from_float<TO>(v);
-  }
+  // A wave a head (query heads first, then key heads with their values), lanes over the head's pairs and then over what
+  // does not turn: both members of a pair come from one lane, which reads each of its numbers once.
+  const int turned = 2 * a.nf, lane = threadIdx.x & 63;
+  const int wave = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6), waves = gridDim.y * (blockDim.x >> 6);
   const int slot = a.slots[t];
   const size_t pg = slot / a.page, off = slot % a.page;
+  TO* __restrict__ qo = (TO*)a.q_out + (size_t)t * a.Hq * a.P;
   TO* __restrict__ kc = (TO*)a.k_cache;
   TO* __restrict__ vc = (TO*)a.v_cache;
   const float* __restrict__ vals = a.v_col < 0 ? k : row + a.v_col;
-  for (int e = first; e < a.Hkv * a.P; e += stride) {
-    const int g = e / a.P, d = e - g * a.P;
-    const float kv = d < a.dim ? value(k, a.k_norm, rk, g, d) : 0.f;
-    kc[((pg * a.Hkv + g) * a.page + off) * a.P + d] = from_float<TO>(kv);
-    const float vv = d < a.vdim ? vals[g * a.vdim + d] : 0.f;
-    vc[((pg * a.Hkv + g) * a.P + d) * a.page + off] = from_float<TO>(vv);
+  for (int job = wave; job < a.Hq + a.Hkv; job += waves) {
+    const bool is_q = job < a.Hq;
+    const int h = is_q ? job : job - a.Hq;
+    const float* __restrict__ x = (is_q ? q : k) + (size_t)h * a.dim;
+    const float* __restrict__ w = is_q ? a.q_norm : a.k_norm;
+    if (w) w += (size_t)h * a.dim;
+    const float r = is_q ? rq : rk;
+    const float mult = is_q && a.q_head_scale ? a.q_head_scale[h] : 1.f;
+    TO* __restrict__ dst = is_q ? qo + (size_t)h * a.P : kc + ((pg * a.Hkv + h) * a.page + off) * a.P;
+    for (int i = lane; i < a.nf; i += 64) {
+      const int d1 = a.layout == LAYOUT_INTERLEAVED ? 2 * i : i, d2 = a.layout == LAYOUT_INTERLEAVED ? 2 * i + 1 : i + a.nf;
+      const float x1 = w ? x[d1] * r * w[d1] : x[d1], x2 = w ? x[d2] * r * w[d2] : x[d2];
+      float o1, o2;
+      rotate_pair(x1, x2, cs[i], cs[a.nf + i], o1, o2);
+      dst[d1] = from_float<TO>(o1 * mult);
+      dst[d2] = from_float<TO>(o2 * mult);
+    }
+    for (int d = turned + lane; d < a.P; d += 64) {
+      const float v = d < a.dim ? (w ? x[d] * r * w[d] : x[d]) * mult : 0.f;
+      dst[d] = from_float<TO>(v);
+    }
+    if (!is_q) {
+      const float* __restrict__ vh = vals + (size_t)h * a.vdim;
+      TO* __restrict__ vd = vc + (pg * a.Hkv + h) * a.P * a.page + off;
+      for (int d = lane; d < a.P; d += 64) vd[(size_t)d * a.page] = from_float<TO>(d < a.vdim ? vh[d] : 0.f);
+    }
   }
 }
 
@@ -120,8 +103,7 @@ MIE_EXPORT int mie_qkv_finish(const float* sums, long ld, int q_col, int k_col, 
                q_out, k_cache, v_cache, Hq, Hkv, dim, vdim, P, page};
   const size_t lds = (size_t)2 * (nf > 0 ? nf : 1) * sizeof(float);
   // few tokens: several workgroups a token, so that a decode step's few rows are spread over the GPU
-  const long numbers = (long)(Hq + Hkv) * P;
-  int parts = tokens >= 256 ? 1 : (int)((numbers + 511) / 512);
+  int parts = tokens >= 256 ? 1 : (Hq + Hkv + 3) / 4;
   parts = parts < 1 ? 1 : parts > 8 ? 8 : parts;
   if (dtype == MIE_F32) hipLaunchKernelGGL(qkv_finish_kernel<float>, dim3(tokens, parts), dim3(256), lds, s, a);
   else if (dtype == MIE_BF16) hipLaunchKernelGGL(qkv_finish_kernel<bf16>, dim3(tokens, parts), dim3(256), lds, s, a);

@@ -479,7 +479,7 @@ __device__ __forceinline__ void store4(bf16* p, float a, float b, float c, float
 template <typename TO, int K>
 __global__ void __launch_bounds__(NORM_THREADS)
 norm_pair_conv_vec_kernel(const float* __restrict__ stream, const float* __restrict__ w1, const float* __restrict__ w2,
-                          const float* __restrict__ taps, const float* __restrict__ tail, const int* __restrict__ token_row,
+                          const float* __restrict__ taps, float* __restrict__ tail, const int* __restrict__ token_row,
                           const int* __restrict__ row_start, const int* __restrict__ slots, TO* __restrict__ xm,
                           TO* __restrict__ y, float* __restrict__ rstd_out, int width, float eps) {
   __shared__ float scratch[16];
@@ -508,7 +508,7 @@ norm_pair_conv_vec_kernel(const float* __restrict__ stream, const float* __restr
   for (int b = 0; b < K; ++b)
     rstd[b] = b <= have ? 1.0f / sqrtf(block_sum(ss[b], scratch) / (float)width + eps) : 0.f;    // ``have`` is the workgroup's
   if (threadIdx.x == 0) rstd_out[t] = rstd[0];
-  const float4* tl = reinterpret_cast<const float4*>(tail + (size_t)slots[r] * (K > 1 ? K - 1 : 1) * width);
+  float4* tl = reinterpret_cast<float4*>(tail + (size_t)slots[r] * (K > 1 ? K - 1 : 1) * width);
 #pragma unroll
   for (int k = 0; k < NPC_V; ++k) {
     const int i = threadIdx.x + k * NORM_THREADS;
@@ -544,15 +544,31 @@ norm_pair_conv_vec_kernel(const float* __restrict__ stream, const float* __restr
              xo[k].w * rstd[0] * g2.w);
     }
   }
+  // A row of one token is this workgroup's alone: it moves the tail on itself (every thread shifts the channels it has
+  // just read, oldest first), and norm_conv_tail_kernel skips such rows.
+  if (K > 1 && row_start[r + 1] - row_start[r] == 1) {
+    float4* tw = tl;
+#pragma unroll
+    for (int k = 0; k < NPC_V; ++k) {
+      const int i = threadIdx.x + k * NORM_THREADS;
+      if (i >= nv) continue;
+      const float4 g = reinterpret_cast<const float4*>(w1)[i];
+#pragma unroll
+      for (int b = 0; b + 2 < K; ++b) tw[(size_t)b * nv + i] = tw[(size_t)(b + 1) * nv + i];
+      tw[(size_t)(K - 2) * nv + i] = make_float4(xo[k].x * rstd[0] * g.x, xo[k].y * rstd[0] * g.y, xo[k].z * rstd[0] * g.z,
+                                                  xo[k].w * rstd[0] * g.w);
+    }
+  }
 }
 
 __global__ void __launch_bounds__(256)
 norm_conv_tail_kernel(const float* __restrict__ stream, const float* __restrict__ w1, const float* __restrict__ rstd,
                       float* __restrict__ tail, const int* __restrict__ row_start, const int* __restrict__ slots, int width,
-                      int K) {
+                      int K, int skip_single) {
   const int r = blockIdx.x, c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= width) return;
   const int a0 = row_start[r], n = row_start[r + 1] - a0, keep = K - 1;
+  if (n == 1 && skip_single) return;           // the row's own workgroup has moved its tail on
   float* tl = tail + (size_t)slots[r] * keep * width;
   for (int i = 0; i < keep; ++i) {
     const int src = n + i;                     // place in the joined sequence of keep + n inputs
@@ -572,7 +588,8 @@ MIE_EXPORT int mie_norm_pair_conv(const float* stream, const float* w1, const fl
   if (out_dtype != MIE_F32 && out_dtype != MIE_BF16) MIE_FAIL("norm_pair_conv: out dtype code %d", out_dtype);
   const bool aligned = !(((uintptr_t)stream | (uintptr_t)w1 | (uintptr_t)w2 | (uintptr_t)taps | (uintptr_t)tail | (uintptr_t)xm |
                           (uintptr_t)y) & 15);
-  if (width % 4 == 0 && width <= 4 * NPC_V * NORM_THREADS && aligned) {
+  const bool vec = width % 4 == 0 && width <= 4 * NPC_V * NORM_THREADS && aligned;    // that kernel moves single-token rows' tails itself
+  if (vec) {
 #define NPC_LAUNCH(TO_, K_)                                                                                                   \
   hipLaunchKernelGGL((norm_pair_conv_vec_kernel<TO_, K_>), dim3(tokens), dim3(NORM_THREADS), 0, s, stream, w1, w2, taps, tail, \
                      token_row, row_start, slots, (TO_*)xm, (TO_*)y, rstd, width, eps)
@@ -592,9 +609,9 @@ MIE_EXPORT int mie_norm_pair_conv(const float* stream, const float* w1, const fl
     hipLaunchKernelGGL(norm_pair_conv_kernel<bf16>, dim3(tokens), dim3(NORM_THREADS), 0, s, stream, w1, w2, taps, tail, token_row,
                        row_start, slots, (bf16*)xm, (bf16*)y, rstd, width, K, eps);
   MIE_CHECK_LAUNCH("norm_pair_conv");
-  if (K > 1) {
+  if (K > 1 && !(vec && tokens == rows)) {
     hipLaunchKernelGGL(norm_conv_tail_kernel, dim3(rows, (width + 255) / 256), dim3(256), 0, s, stream, w1, rstd, tail, row_start,
-                       slots, width, K);
+                       slots, width, K, (int)vec);
     MIE_CHECK_LAUNCH("norm_pair_conv (tail)");
   }
   return 0;
