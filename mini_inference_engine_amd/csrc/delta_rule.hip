@@ -337,6 +337,7 @@ MIE_EXPORT int mie_delta_rule(const float* sums, long ld, int r_col, int k_col, 
   if (tokens <= 0 || rows <= 0) return 0;
   if (H <= 0 || d <= 0 || d > 256 || rank <= 0) MIE_FAIL("delta_rule: %d heads of %d, inner size %d (heads up to 256)", H, d, rank);
   if (H > 65535) MIE_FAIL("delta_rule: %d heads is beyond the grid", H);
+  if (chunk_tokens > 0 && d > 128) MIE_FAIL("delta_rule: heads of %d run whole, not in chunks (up to 128)", d);
   if (chunk_tokens < 0 || (chunk_tokens > 0 && (max_chunks < 1 || !summaries || !starts)))
     MIE_FAIL("delta_rule: chunks of %d tokens, %d a row, need their scratch", chunk_tokens, max_chunks);
   const int heads_here = 255 / d + 2;           // heads a workgroup's 256 channels can touch

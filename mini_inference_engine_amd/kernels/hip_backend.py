@@ -735,6 +735,7 @@ class HipBackend(KernelBackend):
 
     LAYOUTS = {"interleaved": 0, "half": 1}
     DELTA_CHUNK = 64         # tokens a chunk of the delta rule's scan; rows up to this long run whole
+    DELTA_CHUNKED_MAX_DIM = 128   # wider heads always run whole (the fold keeps a chunk's d x d matrix in the LDS)
 
     def qkv_finish(self, sums, q_col, k_col, v_col, num_q_heads, num_kv_heads, dim, vdim, padded_dim, positions, inv_freq,
                    layout, k_cache, v_cache, slot_mapping, q_norm=None, k_norm=None, eps=0.0, q_head_scale=None):
@@ -808,7 +809,7 @@ class HipBackend(KernelBackend):
         prep = torch.empty((T, 3 * n), dtype=torch.float32, device=sums.device)
         longest = int(getattr(step, "max_row_tokens", 0) or (step.host["row_start"][1:] - step.host["row_start"][:-1]).max())
         chunk, chunks, summaries, starts = 0, 0, None, None
-        if longest > self.DELTA_CHUNK and not self.true_fp32:
+        if longest > self.DELTA_CHUNK and not self.true_fp32 and d <= self.DELTA_CHUNKED_MAX_DIM:
             # rows of many tokens: chunks side by side (whether a step takes this path depends on its longest row alone;
             # the two paths differ by the rounding of the fold over whole chunks, so the 32-bit mode keeps to one)
             chunk, chunks = self.DELTA_CHUNK, -(-longest // self.DELTA_CHUNK)

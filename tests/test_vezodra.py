@@ -565,7 +565,9 @@ def test_delta_rule_kernel(hip, dtype):
     for (H, d, rank, lens, slots) in ((2, 16, 8, [1, 1, 9, 2, 70], [4, 1, 3, 5, 2]), (1, 32, 3, [5, 1], [1, 2]), (5, 12, 5, [3, 2, 40], [2, 3, 1]),
                                       (3, 8, 5, [33], [5]), (2, 64, 16, [1, 20], [1, 2]), (1, 128, 4, [6], [3]), (1, 144, 4, [3, 1], [3, 1]),
                                       # rows beyond 64 tokens: the bfloat16 mode runs them in chunks of 64 side by side
-                                      (2, 64, 8, [1, 64, 65, 300, 128], [5, 4, 3, 2, 1]), (3, 24, 4, [129, 2], [1, 2]), (1, 80, 4, [70], [2])):
+                                      (2, 64, 8, [1, 64, 65, 300, 128], [5, 4, 3, 2, 1]), (3, 24, 4, [129, 2], [1, 2]), (1, 80, 4, [70], [2]),
+                                      # inner sizes beyond what the prepare kernel keeps in registers, and no multiple of 4; the widest heads
+                                      (2, 16, 70, [3, 1, 20], [1, 2, 3]), (1, 32, 128, [2, 90], [4, 5]), (1, 200, 6, [5, 1, 66], [1, 2, 3]), (1, 128, 6, [130, 3], [1, 2])):
         step = FakeStep(lens, slots)
         T, n = step.num_tokens, H * d
         cols = dict(r=2, k=2 + n, v=3 + 2 * n, g=3 + 3 * n, a=4 + 4 * n, w=4 + 5 * n)
