@@ -2,9 +2,9 @@
 // C [M, N], for any mix of float and bfloat16 operands, accumulated in true 32-bit FMAs.
 //
 // This is the kernel of the float32 path and the fallback for operand mixes the fast
-// bfloat16 kernels do not take.  Every output element is one accumulator that adds its K
-// products in increasing k, whatever M, N and the tile it falls in are: a token's result
-// is bit-identical however the batch around it is cut.
+// bfloat16 kernels do not take.  Every output element adds its K products in increasing k, sixteen
+// at a time into a partial sum that then joins the total, whatever M, N and the tile it falls in
+// are: a token's result is bit-identical however the batch around it is cut.
 // Also here: silu(gate) * up on the fused gate/up projection output.
 #include "common.hpp"
 
@@ -42,6 +42,13 @@ gemm_nt_kernel(const TA* __restrict__ A, long lda, const TW* __restrict__ W, lon
       Ws[c][r] = w;
     }
     __syncthreads();
+    // the stage's GK products are summed by themselves and then added to the total: the rounding error of a long sum
+    // grows with GK + K / GK terms, not with K
+    float part[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) part[i][j] = 0.f;
 #pragma unroll
     for (int kk = 0; kk < GK; ++kk) {
       float a[4], b[4];
@@ -52,8 +59,12 @@ gemm_nt_kernel(const TA* __restrict__ A, long lda, const TW* __restrict__ W, lon
 #pragma unroll
       for (int i = 0; i < 4; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        for (int j = 0; j < 4; ++j) part[i][j] = fmaf(a[i], b[j], part[i][j]);
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] += part[i][j];
     __syncthreads();
   }
 #pragma unroll
